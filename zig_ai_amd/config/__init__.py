@@ -17,6 +17,7 @@ from .spec import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec, Stream
 from .lfm2 import Lfm2Config, feed_forward_width  # noqa: F401
 from .rudilix import RudilixConfig  # noqa: F401
 from .ranesun import RanesunConfig  # noqa: F401
+from .gemodra import GemodraConfig  # noqa: F401
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -68,3 +69,4 @@ def load_config(model_dir: str):
 register_architecture("Lfm2ForCausalLM", Lfm2Config)
 register_architecture("Rudilix", RudilixConfig)
 register_architecture("Ranesun", RanesunConfig)
+register_architecture("Gemodra", GemodraConfig)

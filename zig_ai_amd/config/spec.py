@@ -67,7 +67,7 @@ class LayerSpec:
 
 @dataclass(frozen=True)
 class StreamStep:
-    """Something that enters the residual stream right before a run-order entry:
+    """Something that enters the residual stream right before or right after a run-order entry:
     ``part`` indexes ``ModelSpec.stream_parts``, ``args`` are the keywords its ``forward``
     gets at this place (which row of its table, say)."""
 
@@ -84,13 +84,16 @@ class LayerCall:
     calls with ``writes_cache`` store into it (a reader of another layer's
     cache has ``writes_cache=False``).  ``cache=None`` gives the call an entry
     of its own (a layer that the run order names several times then has a cache,
-    or a state, per time it runs).  ``before``: see ``StreamStep``.
+    or a state, per time it runs).  ``before`` / ``after``: see ``StreamStep``; ``after``
+    runs once the entry's block has returned, so what diagnostics call the stream after
+    the entry holds it.
     """
 
     layer: int
     cache: Optional[int] = None
     writes_cache: bool = True
     before: Optional[StreamStep] = None
+    after: Optional[StreamStep] = None
 
 
 @dataclass(frozen=True)
@@ -116,9 +119,10 @@ class ModelSpec:
             if not 0 <= call.layer < len(self.layers):
                 raise ConfigError(
                     f"run order names layer {call.layer}, but there are {len(self.layers)} layers")
-            if call.before is not None and not 0 <= call.before.part < len(self.stream_parts):
-                raise ConfigError(f"run order names stream part {call.before.part}, but there are "
-                                  f"{len(self.stream_parts)}")
+            for named in (call.before, call.after):
+                if named is not None and not 0 <= named.part < len(self.stream_parts):
+                    raise ConfigError(f"run order names stream part {named.part}, but there are "
+                                      f"{len(self.stream_parts)}")
 
     def resolved_schedule(self) -> Tuple[LayerCall, ...]:
         """The run order with every ``cache=None`` replaced by a fresh id."""
@@ -130,7 +134,7 @@ class ModelSpec:
                 while next_id in used:
                     next_id += 1
                 used.add(next_id)
-                out.append(LayerCall(call.layer, next_id, call.writes_cache, call.before))
+                out.append(LayerCall(call.layer, next_id, call.writes_cache, call.before, call.after))
             else:
                 out.append(call)
         return tuple(out)

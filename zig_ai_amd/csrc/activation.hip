@@ -256,3 +256,54 @@ extern "C" int za_scale(float* x, float s, long long n, hipStream_t stream) {
                      (size_t)n);
   return za_launch_status();
 }
+
+// x <- cap * tanh(x / cap), 32-bit, in place (an output head's cap on its logits).
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ x, float cap, size_t n) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < n) x[idx] = cap * tanhf(x[idx] / cap);
+}
+
+extern "C" int za_softcap(float* x, float cap, long long n, hipStream_t stream) {
+  if (n == 0) return 0;
+  if (n < 0 || !x || !(cap > 0.f)) return ZA_ERR_ARG;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x,
+                     cap, (size_t)n);
+  return za_launch_status();
+}
+
+// out[t][j] = act(g[t][j]) * table[ids[t]][col0 + j]: a gate (computed from something
+// else) on a slice of a table row that the token's id picks.  `table` has `ld` columns
+// and `rows` rows; an id outside the table yields zeros.
+template <typename T, typename TT>
+__global__ void __launch_bounds__(256)
+table_gate_kernel(const T* __restrict__ g, const int* __restrict__ ids,
+                  const TT* __restrict__ table, int rows, int ld, int col0, T* __restrict__ out,
+                  int n_tokens, int dim, int act) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)n_tokens * dim) return;
+  const size_t t = idx / dim;
+  const int j = (int)(idx % dim), id = ids[t];
+  const float e = (id >= 0 && id < rows) ? to_f32<TT>(table[(size_t)id * ld + col0 + j]) : 0.f;
+  out[idx] = from_f32<T>(gate_act(to_f32<T>(g[idx]), act) * e);
+}
+
+// dtype codes: 0 = float32, 1 = bfloat16 (of g and out; the table has its own)
+extern "C" int za_table_gate(const void* g, int dtype, const int* ids, const void* table,
+                             int table_dtype, int rows, int ld, int col0, void* out, int n_tokens,
+                             int dim, int act, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || dim <= 0 || !g || !ids || !table || !out || rows <= 0 || col0 < 0 ||
+      col0 + dim > ld || act < 0 || act > 1)
+    return ZA_ERR_ARG;
+  dim3 grid((unsigned)(((size_t)n_tokens * dim + 255) / 256)), block(256);
+#define ZA_TG(T, TT)                                                                            \
+  hipLaunchKernelGGL((table_gate_kernel<T, TT>), grid, block, 0, stream, (const T*)g, ids,      \
+                     (const TT*)table, rows, ld, col0, (T*)out, n_tokens, dim, act)
+  if (dtype == 0 && table_dtype == 0) ZA_TG(float, float);
+  else if (dtype == 0 && table_dtype == 1) ZA_TG(float, bf16_t);
+  else if (dtype == 1 && table_dtype == 1) ZA_TG(bf16_t, bf16_t);
+  else if (dtype == 1 && table_dtype == 0) ZA_TG(bf16_t, float);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_TG
+  return za_launch_status();
+}

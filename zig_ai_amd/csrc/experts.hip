@@ -407,3 +407,171 @@ extern "C" int za_grouped_gemm(const void* src, int src_dtype, long long src_row
 #undef ZA_GF
   return za_launch_status();
 }
+
+// ------------------------------------------------------------------------ a router
+// Which `top` of `n` router outputs every token uses, and with which weight.  One wave a
+// token, everything in 32-bit:
+//   s = softmax(z) over all n outputs (mode 0) or sigmoid(z) (mode 1)
+//   c = s + correction          the choice score (correction may be absent)
+//   the outputs form `groups` equal groups of neighbours; a group's score is its largest c,
+//   and only outputs of the `keep` best groups can be chosen (the others count as minus
+//   infinity); groups == 0: no such limit
+//   chosen = the `top` outputs with the largest c, in descending order (of equal scores the
+//   lower index first); weight = s[chosen] * scale, or, `renorm`, divided by the sum of
+//   the chosen s first
+// What an output beyond the experts that have weights means (an expert that hands its input
+// on, say) is the business of whoever reads `chosen`.
+#define RT_MAX 1024
+
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int o = ZA_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, ZA_WAVE);
+    const int oi = __shfl_xor(i, o, ZA_WAVE);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+}
+
+__global__ void __launch_bounds__(64)
+route_topk_kernel(const float* __restrict__ z, int ld, const float* __restrict__ correction, int n,
+                  int groups, int keep, int top, float scale, int mode, int renorm,
+                  int* __restrict__ chosen, float* __restrict__ weight) {
+  __shared__ float ss[RT_MAX], cs[RT_MAX], gs[RT_MAX];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* zr = z + (size_t)t * ld;
+  if (mode == 0) {
+    float mx = -INFINITY;
+    for (int e = lane; e < n; e += 64) mx = fmaxf(mx, zr[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < n; e += 64) {
+      const float p = expf(zr[e] - mx);
+      ss[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < n; e += 64) ss[e] *= inv;
+  } else {
+    for (int e = lane; e < n; e += 64) ss[e] = 1.0f / (1.0f + expf(-zr[e]));
+  }
+  for (int e = lane; e < n; e += 64) cs[e] = ss[e] + (correction ? correction[e] : 0.f);
+  __builtin_amdgcn_wave_barrier();
+  __syncthreads();
+  if (groups > 1 && keep < groups) {
+    const int per = n / groups;
+    for (int g = lane; g < groups; g += 64) {
+      float best = -INFINITY;
+      for (int k = 0; k < per; ++k) best = fmaxf(best, cs[g * per + k]);
+      gs[g] = best;
+    }
+    __syncthreads();
+    // the `keep` best groups get the mark +inf; afterwards every other group is closed
+    for (int r = 0; r < keep; ++r) {
+      float v = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += 64) {
+        const float x = gs[g];
+        if (x != INFINITY && (x > v || (x == v && g < at))) { v = x; at = g; }
+      }
+      wave_argmax(v, at);
+      __syncthreads();
+      if (lane == 0 && at < groups) gs[at] = INFINITY;
+      __syncthreads();
+    }
+    for (int e = lane; e < n; e += 64)
+      if (gs[e / per] != INFINITY) cs[e] = -INFINITY;
+    __syncthreads();
+  }
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float v = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < n; e += 64) {
+      const float x = cs[e];
+      // (a taken output holds NaN, which compares false)
+      if (x > v || (x == v && e < at)) { v = x; at = e; }
+    }
+    wave_argmax(v, at);
+    __syncthreads();
+    if (at >= n) at = 0;      // nothing left to choose from: cannot happen with top <= open outputs
+    const float s = ss[at];
+    total += s;
+    if (lane == 0) {
+      chosen[(size_t)t * top + j] = at;
+      weight[(size_t)t * top + j] = s;
+      cs[at] = __builtin_nanf("");
+    }
+    __syncthreads();
+  }
+  const float f = renorm ? scale / total : scale;
+  for (int j = lane; j < top; j += 64) weight[(size_t)t * top + j] *= f;
+}
+
+extern "C" int za_route_topk(const float* z, int ld, const float* correction, int n_tokens, int n,
+                             int groups, int keep, int top, float scale, int mode, int renorm,
+                             int* chosen, float* weight, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || n <= 0 || ld < n || top <= 0 || top > n || !z || !chosen || !weight ||
+      groups < 0 || (groups > 0 && (n % groups != 0 || keep <= 0 || keep > groups)) ||
+      mode < 0 || mode > 1)
+    return ZA_ERR_ARG;
+  if (groups > 0 && (long long)keep * (n / groups) < top) return ZA_ERR_ARG;
+  if (n > RT_MAX) return ZA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(route_topk_kernel, dim3(n_tokens), dim3(64), 0, stream, z, ld, correction, n,
+                     groups, keep, top, scale, mode, renorm, chosen, weight);
+  return za_launch_status();
+}
+
+// What a token's chosen experts and the shared expert give, as one 32-bit row:
+//   y[t] = sum_j weight[t][j] * (chosen[t][j] < n_real ? expert_out[t * top + j] : x[t])
+//          + gate(t) * shared[t]
+// An output beyond the n_real experts that have weights hands the token's input x[t] on.
+// gate(t) = sigmoid(gate_logits[t * gate_ld]) when gate_logits is given, else 1; `shared`
+// may be absent.  The sum is taken in the order j = 0 .. top - 1, then the shared expert.
+template <typename TE, typename TX>
+__global__ void __launch_bounds__(256)
+experts_combine_kernel(const TE* __restrict__ expert_out, const int* __restrict__ chosen,
+                       const float* __restrict__ weight, const TX* __restrict__ x,
+                       const TE* __restrict__ shared, const float* __restrict__ gate_logits,
+                       int gate_ld, float* __restrict__ y, int top, int n_real, int width) {
+  const size_t t = blockIdx.x;
+  float g = 1.0f;
+  if (shared && gate_logits) g = 1.0f / (1.0f + expf(-gate_logits[t * gate_ld]));
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const int e = chosen[t * top + j];
+      const float w = weight[t * top + j];
+      const float v = e < n_real ? to_f32<TE>(expert_out[(t * top + j) * width + i])
+                                 : to_f32<TX>(x[t * width + i]);
+      acc = fmaf(w, v, acc);
+    }
+    if (shared) acc = fmaf(g, to_f32<TE>(shared[t * width + i]), acc);
+    y[t * width + i] = acc;
+  }
+}
+
+// dtype codes: 0 = float32, 1 = bfloat16; `out_dtype` is that of expert_out and shared.
+extern "C" int za_experts_combine(const void* expert_out, int out_dtype, const int* chosen,
+                                  const float* weight, const void* x, int x_dtype,
+                                  const void* shared, const float* gate_logits, int gate_ld,
+                                  float* y, int n_tokens, int top, int n_real, int width,
+                                  hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || top <= 0 || width <= 0 || n_real < 0 || !chosen || !weight || !x || !y ||
+      (n_real > 0 && !expert_out))
+    return ZA_ERR_ARG;
+  dim3 grid(n_tokens), block(width <= 256 ? 64 : 256);
+#define ZA_EC(TE, TX)                                                                          \
+  hipLaunchKernelGGL((experts_combine_kernel<TE, TX>), grid, block, 0, stream,                 \
+                     (const TE*)expert_out, chosen, weight, (const TX*)x, (const TE*)shared,   \
+                     gate_logits, gate_ld, y, top, n_real, width)
+  if (out_dtype == 0 && x_dtype == 0) ZA_EC(float, float);
+  else if (out_dtype == 0 && x_dtype == 1) ZA_EC(float, bf16_t);
+  else if (out_dtype == 1 && x_dtype == 1) ZA_EC(bf16_t, bf16_t);
+  else if (out_dtype == 1 && x_dtype == 0) ZA_EC(bf16_t, float);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_EC
+  return za_launch_status();
+}

@@ -1,0 +1,612 @@
+// Attention over one small latent vector a token ("latent attention"): what is cached for
+// a token is a normed latent c [R] and, optionally, a rotated key part k_r [Dr] that all
+// heads share; every head's keys and values are linear expansions of c,
+//     k_h = Wuk_h c,   v_h = Wuv_h c.
+// Neither is ever formed.  With q_h = [q_n | q_r] (unrotated | rotated),
+//     q_h . [k_h | k_r] = (Wuk_h^T q_n) . c + q_r . k_r
+//     sum_j p_j v_h,j   = Wuv_h (sum_j p_j c_j)
+// so the attention runs with ONE key/value head whose key is the cached row [c | k_r]
+// (W = R + Dr elements) and whose value is the row's first R elements, with queries
+// [Wuk_h^T q_n | q_r] and results that the head's Wuv expands afterwards.  The cache holds
+// one plane of W elements a token, rows of a page one after the other.
+//
+// Kernels:
+//   latent_prepare     a token's opening projection -> the normed query latent, and the row
+//                      [rmsnorm(c) | rotate(k_r)] into the token's place in the cache
+//   rotate_part        the rotated part of every head's query into the folded query
+//   head_linear        out[t][h] = x[t][h] @ W[h]^T for every head at once (the two
+//                      foldings above), optionally times sigmoid(gate) a head or an element
+//   latent_attention   the attention itself: causal, streaming softmax in 32-bit with a sink
+//                      a head, any mix of prompt portions and single tokens in one launch,
+//                      contexts optionally cut into ranges (latent_combine merges them)
+//   latent_attention_mfma   the same on the matrix cores (bfloat16)
+// Rotation: adjacent pairs (2i, 2i + 1) or halves (i, i + dims/2) of the first `rot_dims`
+// elements, angle = position * inv_freq[i] in 32-bit.
+#include <math.h>
+
+#include "common.h"
+
+// ------------------------------------------------------------------ latent_prepare
+// down: [T][ld], columns [q_col, q_col + Rq) the query latent, [c_col, c_col + R) the
+// latent, then Dr elements of the rotated key part.  cq: [T][Rq].  plane: the cache,
+// token t's row at plane + (slots[t] / page_size) * page_stride + (slots[t] % page_size) * W.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_prepare_kernel(const T* __restrict__ down, int ld, int q_col, int Rq, int c_col, int R,
+                      int Dr, const float* __restrict__ q_norm_w, const float* __restrict__ c_norm_w,
+                      float eps, const int* __restrict__ positions, const int* __restrict__ slots,
+                      const float* __restrict__ inv_freq, int rot_dims, int adjacent,
+                      T* __restrict__ cq, T* __restrict__ plane, int page_size,
+                      long long page_stride) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const T* row = down + t * ld;
+  const int tid = threadIdx.x, bd = blockDim.x;
+  if (cq) {
+    float ss = 0.f;
+    for (int i = tid; i < Rq; i += bd) {
+      const float v = to_f32<T>(row[q_col + i]);
+      ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float f = 1.0f / sqrtf(ss / (float)Rq + eps);
+    for (int i = tid; i < Rq; i += bd)
+      cq[t * Rq + i] = from_f32<T>(to_f32<T>(row[q_col + i]) * f * q_norm_w[i]);
+  }
+  if (!plane) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  T* dst = plane + (size_t)(slot / page_size) * page_stride + (size_t)(slot % page_size) * (R + Dr);
+  float ss = 0.f;
+  for (int i = tid; i < R; i += bd) {
+    const float v = to_f32<T>(row[c_col + i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float f = 1.0f / sqrtf(ss / (float)R + eps);
+  for (int i = tid; i < R; i += bd)
+    dst[i] = from_f32<T>(to_f32<T>(row[c_col + i]) * f * c_norm_w[i]);
+  const T* kr = row + c_col + R;
+  const int half = rot_dims / 2;
+  const float pos = (float)positions[t];
+  for (int i = tid; i < half; i += bd) {
+    const int a = adjacent ? 2 * i : i, b = adjacent ? 2 * i + 1 : i + half;
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    const float u = to_f32<T>(kr[a]), v = to_f32<T>(kr[b]);
+    dst[R + a] = from_f32<T>(u * cs - v * sn);
+    dst[R + b] = from_f32<T>(v * cs + u * sn);
+  }
+  for (int i = rot_dims + tid; i < Dr; i += bd) dst[R + i] = kr[i];
+}
+
+extern "C" int za_latent_prepare(const void* down, int dtype, int ld, int q_col, int q_rank,
+                                 int c_col, int kv_rank, int rot_dim, const float* q_norm_w,
+                                 const float* c_norm_w, float eps, const int* positions,
+                                 const int* slots, const float* inv_freq, int rot_dims,
+                                 int adjacent, void* cq, void* plane, int page_size,
+                                 long long page_stride, int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || !down || ld <= 0 || kv_rank <= 0 || rot_dim < 0 || rot_dims < 0 ||
+      rot_dims > rot_dim || rot_dims % 2 != 0 || c_col < 0 || c_col + kv_rank + rot_dim > ld ||
+      (cq && (q_rank <= 0 || q_col < 0 || q_col + q_rank > ld || !q_norm_w)) ||
+      (plane && (!slots || !c_norm_w || page_size <= 0 || page_stride < (long long)page_size * (kv_rank + rot_dim))) ||
+      (plane && rot_dims > 0 && (!inv_freq || !positions)))
+    return ZA_ERR_ARG;
+  dim3 grid(n_tokens), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL((latent_prepare_kernel<float>), grid, block, 0, stream, (const float*)down,
+                       ld, q_col, q_rank, c_col, kv_rank, rot_dim, q_norm_w, c_norm_w, eps,
+                       positions, slots, inv_freq, rot_dims, adjacent, (float*)cq, (float*)plane,
+                       page_size, page_stride);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((latent_prepare_kernel<bf16_t>), grid, block, 0, stream,
+                       (const bf16_t*)down, ld, q_col, q_rank, c_col, kv_rank, rot_dim, q_norm_w,
+                       c_norm_w, eps, positions, slots, inv_freq, rot_dims, adjacent, (bf16_t*)cq,
+                       (bf16_t*)plane, page_size, page_stride);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}
+
+// --------------------------------------------------------------------- rotate_part
+// dst[t][h][dst_col + i] = rotation of src[t][h][src_col + i], i < Dr (elements beyond
+// rot_dims are copied).  One thread a pair.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rotate_part_kernel(const T* __restrict__ src, int src_ld, int src_col, T* __restrict__ dst,
+                   int dst_ld, int dst_col, int H, int Dr, const int* __restrict__ positions,
+                   const float* __restrict__ inv_freq, int rot_dims, int adjacent, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int per = Dr - rot_dims / 2;         // pairs, then the elements that pass unchanged
+  const size_t th = idx / per;               // token * H + head
+  const int i = (int)(idx % per);
+  const T* s = src + th * src_ld + src_col;
+  T* d = dst + th * dst_ld + dst_col;
+  const int half = rot_dims / 2;
+  if (i < half) {
+    const int a = adjacent ? 2 * i : i, b = adjacent ? 2 * i + 1 : i + half;
+    float sn, cs;
+    sincosf((float)positions[th / H] * inv_freq[i], &sn, &cs);
+    const float u = to_f32<T>(s[a]), v = to_f32<T>(s[b]);
+    d[a] = from_f32<T>(u * cs - v * sn);
+    d[b] = from_f32<T>(v * cs + u * sn);
+  } else {
+    const int e = rot_dims + (i - half);
+    d[e] = s[e];
+  }
+}
+
+extern "C" int za_rotate_part(const void* src, int dtype, int src_ld, int src_col, void* dst,
+                              int dst_ld, int dst_col, int n_tokens, int heads, int rot_dim,
+                              const int* positions, const float* inv_freq, int rot_dims,
+                              int adjacent, hipStream_t stream) {
+  if (n_tokens == 0 || rot_dim == 0) return 0;
+  if (n_tokens < 0 || heads <= 0 || rot_dim < 0 || rot_dims < 0 || rot_dims > rot_dim ||
+      rot_dims % 2 != 0 || !src || !dst || src_col < 0 || dst_col < 0 ||
+      src_col + rot_dim > src_ld || dst_col + rot_dim > dst_ld ||
+      (rot_dims > 0 && (!positions || !inv_freq)))
+    return ZA_ERR_ARG;
+  const size_t total = (size_t)n_tokens * heads * (rot_dim - rot_dims / 2);
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL((rotate_part_kernel<float>), grid, block, 0, stream, (const float*)src,
+                       src_ld, src_col, (float*)dst, dst_ld, dst_col, heads, rot_dim, positions,
+                       inv_freq, rot_dims, adjacent, total);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((rotate_part_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)src,
+                       src_ld, src_col, (bf16_t*)dst, dst_ld, dst_col, heads, rot_dim, positions,
+                       inv_freq, rot_dims, adjacent, total);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}
+
+// --------------------------------------------------------------------- head_linear
+// out[t][h][o_col + n] = (sum_k x[t][h][x_col + k] * W[h][n][k]) * gate(t, h, n)
+//   x:   [T][H][x_ld]      W: [H][N][K]      out: [T][H][o_ld]
+//   gate_mode 0: none; 1: sigmoid(gate[t][gate_col + h]); 2: sigmoid(gate[t][gate_col + h*N + n])
+// Every output element is a sum over k in an order fixed by K alone.
+struct HeadLinearArgs {
+  const void* x;
+  const void* W;
+  void* out;
+  const void* gate;
+  int T, H, N, K;
+  int x_ld, x_col, o_ld, o_col;
+  int gate_ld, gate_col, gate_mode;
+};
+
+template <typename TG>
+__device__ __forceinline__ float head_gate_of(const HeadLinearArgs& a, int t, int h, int n) {
+  if (a.gate_mode == 0) return 1.0f;
+  const TG* g = (const TG*)a.gate + (size_t)t * a.gate_ld + a.gate_col;
+  const float z = to_f32<TG>(a.gate_mode == 1 ? g[h] : g[(size_t)h * a.N + n]);
+  return 1.0f / (1.0f + expf(-z));
+}
+
+// bfloat16 on the matrix cores, operands straight from memory into the fragments
+// (v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k-slots (l / 16) * 8 .. + 7 of
+// either operand and receives rows (l / 16) * 4 .. + 3, column (l % 16) of the product).
+// TM = 64: four waves of 16 rows x 64 columns; TM = 16 (decode batches): four waves of 16
+// columns each.
+template <int TM, typename TO>
+__global__ void __launch_bounds__(256)
+head_linear_bf16_kernel(HeadLinearArgs a) {
+  constexpr int WM = TM / 16;          // waves along the rows
+  constexpr int WN = 4 / WM;           // waves along the columns
+  constexpr int NT = 4 / WN;           // 16-column tiles a wave
+  const int h = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % WM, wn = wave / WM;
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.y * 64 + wn * NT * 16;
+  const int K = a.K, N = a.N;
+  const int row = blockIdx.x * TM + wm * 16 + r16;
+  const bool row_ok = row < a.T;
+  const bf16_t* arow = (const bf16_t*)a.x + ((size_t)(row_ok ? row : 0) * a.H + h) * a.x_ld + a.x_col;
+  const bf16_t* wbase = (const bf16_t*)a.W + (size_t)h * N * K;
+  const bf16_t* wrow[NT];
+  bool col_ok[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + j * 16 + r16;
+    col_ok[j] = n < N;
+    wrow[j] = wbase + (size_t)(col_ok[j] ? n : 0) * K;
+  }
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int U = 2;
+  for (int k0 = 0; k0 < K; k0 += 32 * U) {
+    bf16x8_t fa[U], fw[U][NT];
+#pragma unroll
+    for (int s = 0; s < U; ++s) {
+      const int k = k0 + s * 32 + kq * 8;
+      const bool k_ok = k < K;           // K is a multiple of 8: a piece is inside or outside
+      fa[s] = (row_ok && k_ok) ? *reinterpret_cast<const bf16x8_t*>(arow + k) : zero;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        fw[s][j] = (col_ok[j] && k_ok) ? *reinterpret_cast<const bf16x8_t*>(wrow[j] + k) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < U; ++s)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s], fw[s][j], acc[j], 0, 0, 0);
+  }
+  TO* out = (TO*)a.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = blockIdx.x * TM + wm * 16 + kq * 4 + i;
+    if (r >= a.T) continue;
+    TO* orow = out + ((size_t)r * a.H + h) * a.o_ld + a.o_col;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int n = n0 + j * 16 + r16;
+      if (n < N) orow[n] = from_f32<TO>(acc[j][i] * head_gate_of<bf16_t>(a, r, h, n));
+    }
+  }
+}
+
+// 32-bit weights (x of either type): 64 x 64 tiles through LDS, plain FMA.
+template <typename TA, typename TO>
+__global__ void __launch_bounds__(256)
+head_linear_f32_kernel(HeadLinearArgs a) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  const int h = blockIdx.z;
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const int n0 = blockIdx.y * 64, m0 = blockIdx.x * 64;
+  const int K = a.K, N = a.N;
+  const float* W = (const float*)a.W + (size_t)h * N * K;
+  const int lrow = tid / 4, lk = (tid % 4) * 4;
+  const bool a_ok = m0 + lrow < a.T;
+  const TA* arow = (const TA*)a.x + ((size_t)(a_ok ? m0 + lrow : 0) * a.H + h) * a.x_ld + a.x_col;
+  const bool w_ok = n0 + lrow < N;
+  const float* wrow = W + (size_t)(w_ok ? n0 + lrow : 0) * K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + lk + j;
+      As[lk + j][lrow] = (a_ok && k < K) ? to_f32<TA>(arow[k]) : 0.f;
+      Ws[lk + j][lrow] = (w_ok && k < K) ? wrow[k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  TO* out = (TO*)a.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = m0 + ty * 4 + i;
+    if (r >= a.T) continue;
+    TO* orow = out + ((size_t)r * a.H + h) * a.o_ld + a.o_col;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) orow[n] = from_f32<TO>(acc[i][j] * head_gate_of<TA>(a, r, h, n));
+    }
+  }
+}
+
+// dtype codes: 0 = float32, 1 = bfloat16.  The gate has x's type.
+extern "C" int za_head_linear(const void* x, int x_dtype, int x_ld, int x_col, const void* W,
+                              int w_dtype, void* out, int out_dtype, int o_ld, int o_col,
+                              int n_tokens, int heads, int N, int K, const void* gate, int gate_ld,
+                              int gate_col, int gate_mode, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || heads <= 0 || heads > 65535 || N <= 0 || K <= 0 || !x || !W || !out ||
+      x_col < 0 || o_col < 0 || x_col + K > x_ld || o_col + N > o_ld || gate_mode < 0 ||
+      gate_mode > 2 || (gate_mode && (!gate || gate_col < 0)) ||
+      (gate_mode == 1 && gate_col + heads > gate_ld) ||
+      (gate_mode == 2 && (long long)gate_col + (long long)heads * N > gate_ld))
+    return ZA_ERR_ARG;
+  HeadLinearArgs a{x, W, out, gate, n_tokens, heads, N, K, x_ld, x_col, o_ld, o_col,
+                   gate_ld, gate_col, gate_mode};
+  const unsigned ntiles = (unsigned)((N + 63) / 64);
+  if (w_dtype == 1) {
+    if (x_dtype != 1 || K % 8 != 0 || x_ld % 8 != 0 || x_col % 8 != 0) return ZA_ERR_UNSUPPORTED;
+    const bool small = n_tokens <= 16;
+    dim3 grid((unsigned)((n_tokens + (small ? 15 : 63)) / (small ? 16 : 64)), ntiles, heads);
+#define ZA_HL(TMM, TO) \
+  hipLaunchKernelGGL((head_linear_bf16_kernel<TMM, TO>), grid, dim3(256), 0, stream, a)
+    if (out_dtype == 0) { if (small) ZA_HL(16, float); else ZA_HL(64, float); }
+    else if (out_dtype == 1) { if (small) ZA_HL(16, bf16_t); else ZA_HL(64, bf16_t); }
+    else return ZA_ERR_UNSUPPORTED;
+#undef ZA_HL
+    return za_launch_status();
+  }
+  if (w_dtype != 0) return ZA_ERR_UNSUPPORTED;
+  dim3 grid((unsigned)((n_tokens + 63) / 64), ntiles, heads);
+#define ZA_HF(TA, TO) \
+  hipLaunchKernelGGL((head_linear_f32_kernel<TA, TO>), grid, dim3(256), 0, stream, a)
+  if (x_dtype == 0 && out_dtype == 0) ZA_HF(float, float);
+  else if (x_dtype == 1 && out_dtype == 0) ZA_HF(bf16_t, float);
+  else if (x_dtype == 1 && out_dtype == 1) ZA_HF(bf16_t, bf16_t);
+  else if (x_dtype == 0 && out_dtype == 1) ZA_HF(float, bf16_t);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_HF
+  return za_launch_status();
+}
+
+// ---------------------------------------------------------------- latent_attention
+// The general kernel: any sizes, 32-bit or bfloat16 storage, everything computed in 32-bit.
+// A workgroup serves one work item (up to `count` consecutive query tokens of one request)
+// and one chunk of up to LA_MAX_ROWS / count heads; a tile of KT cached rows staged in LDS
+// is shared by all of them.  Rows (token, head) are dealt to the four waves; in the score
+// phase a lane owns a key, in the value phase it owns latent elements.  Contexts may be cut
+// into `nsplit` ranges of `keys_per_split` keys, cut at key positions that depend on nothing
+// else; latent_combine merges the partial (maximum, sum, accumulator).  The sink joins the
+// denominator once: at the end of a whole context here, or in the merge.
+#define LA_WAVES 4
+#define LA_RPW 8
+#define LA_MAX_ROWS (LA_WAVES * LA_RPW)
+#define LA_MAX_W 576
+#define LA_MAX_R 512
+#define LA_RPL (LA_MAX_R / 64)        // latent elements per lane, at most
+
+template <typename T, int KT>
+__global__ void __launch_bounds__(256)
+latent_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ plane,
+                        long long page_stride, const int* __restrict__ block_table, int bt_stride,
+                        const int* __restrict__ positions, const int* __restrict__ wi_seq,
+                        const int* __restrict__ wi_row0, const int* __restrict__ wi_count,
+                        float* __restrict__ part_acc, float* __restrict__ part_ml, int H, int HC,
+                        int W, int R, int page_size, float scale, int keys_per_split, int nsplit,
+                        const float* __restrict__ sink) {
+  extern __shared__ float smem[];
+  const int ldk = W + 1;
+  float* Ks = smem;                       // [KT][W + 1]
+  float* Qs = Ks + KT * ldk;              // [LA_MAX_ROWS][W]
+  float* Ps = Qs + LA_MAX_ROWS * W;       // [LA_WAVES][64]
+
+  const int item = blockIdx.x, z = blockIdx.z;
+  const int h0 = blockIdx.y * HC;
+  const int G = min(HC, H - h0);          // heads of this chunk
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int seq = wi_seq[item];
+  const int row0 = wi_row0[item];
+  int count = wi_count[item];
+  if (count * G > LA_MAX_ROWS) count = LA_MAX_ROWS / G;   // the host never asks for more
+  const int rows = count * G;
+  const int* table = block_table + (size_t)seq * bt_stride;
+
+  const int hi = positions[row0 + count - 1];   // inclusive
+  int range_lo = z * keys_per_split;
+  int range_hi = range_lo + keys_per_split - 1;
+  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
+  if (range_hi > hi) range_hi = hi;
+
+  for (int idx = tid; idx < rows * W; idx += 256) {
+    const int r = idx / W, dd = idx % W;
+    const int tok = row0 + r / G, h = h0 + r % G;
+    Qs[r * W + dd] = to_f32<T>(q[((size_t)tok * H + h) * W + dd]);
+  }
+
+  float m[LA_RPW], l[LA_RPW], acc[LA_RPW][LA_RPL];
+#pragma unroll
+  for (int i = 0; i < LA_RPW; ++i) {
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+#pragma unroll
+    for (int c = 0; c < LA_RPL; ++c) acc[i][c] = 0.f;
+  }
+
+  for (int tile0 = range_lo; tile0 <= range_hi; tile0 += KT) {
+    __syncthreads();  // previous tile fully consumed (and Qs written, first time)
+    for (int idx = tid; idx < KT * W; idx += 256) {
+      const int j = idx / W, c = idx % W;
+      const int kp = tile0 + j;
+      float v = 0.f;
+      if (kp <= range_hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          v = to_f32<T>(plane[(size_t)page * page_stride + (size_t)(kp % page_size) * W + c]);
+      }
+      Ks[j * ldk + c] = v;
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int lr = 0; lr < LA_RPW; ++lr) {
+      const int r = wave + LA_WAVES * lr;
+      if (r < rows) {
+        const int pos = positions[row0 + r / G];
+        const int kp = tile0 + lane;
+        const bool valid = lane < KT && kp <= pos && kp <= range_hi;
+        float s = -INFINITY;
+        if (lane < KT) {
+          const float* qr = Qs + r * W;
+          const float* kr = Ks + lane * ldk;
+          float dot = 0.f;
+          for (int dd = 0; dd < W; ++dd) dot = fmaf(qr[dd], kr[dd], dot);
+          if (valid) s = dot * scale;
+        }
+        const float tmax = wave_max(s);
+        const float m_new = fmaxf(m[lr], tmax);
+        if (m_new > -INFINITY) {
+          const float alpha = expf(m[lr] - m_new);
+          const float p = valid ? expf(s - m_new) : 0.f;
+          l[lr] = l[lr] * alpha + wave_sum(p);
+          m[lr] = m_new;
+          __builtin_amdgcn_wave_barrier();
+          Ps[wave * 64 + lane] = p;
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int c = 0; c < LA_RPL; ++c) {
+            const int dd = lane + 64 * c;
+            if (64 * c < R) {
+              float a = acc[lr][c] * alpha;
+              if (dd < R) {
+#pragma unroll 8
+                for (int j = 0; j < KT; ++j) a = fmaf(Ps[wave * 64 + j], Ks[j * ldk + dd], a);
+              }
+              acc[lr][c] = a;
+            }
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int lr = 0; lr < LA_RPW; ++lr) {
+    const int r = wave + LA_WAVES * lr;
+    if (r < rows) {
+      const int tok = row0 + r / G, h = h0 + r % G;
+      if (nsplit == 1) {
+        if (sink) l[lr] += expf(sink[h] - m[lr]);
+        const float inv = l[lr] > 0.f ? 1.0f / l[lr] : 0.f;
+        T* o = out + ((size_t)tok * H + h) * R;
+#pragma unroll
+        for (int c = 0; c < LA_RPL; ++c) {
+          const int dd = lane + 64 * c;
+          if (dd < R) o[dd] = from_f32<T>(acc[lr][c] * inv);
+        }
+      } else {
+        const size_t pidx = ((size_t)tok * H + h) * nsplit + z;
+        float* pa = part_acc + pidx * R;
+#pragma unroll
+        for (int c = 0; c < LA_RPL; ++c) {
+          const int dd = lane + 64 * c;
+          if (dd < R) pa[dd] = acc[lr][c];
+        }
+        if (lane == 0) {
+          part_ml[pidx * 2] = m[lr];
+          part_ml[pidx * 2 + 1] = l[lr];
+        }
+      }
+    }
+  }
+}
+
+// The partial results of a row's ranges -> the row.  `base2`: the partial maxima are whole
+// numbers on the base-2 scale (what the matrix-core kernel keeps), so a partial result's
+// weight 2^(m_z - m) is an exact power of two.
+template <typename T>
+__global__ void __launch_bounds__(64)
+latent_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                      T* __restrict__ out, int R, int nsplit, int base2,
+                      const float* __restrict__ sink, int H) {
+  const size_t row = blockIdx.x;  // token * H + head
+  const int lane = threadIdx.x;
+  float mx = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, part_ml[(row * nsplit + z) * 2]);
+  float total = 0.f;
+  float acc[LA_RPL];
+#pragma unroll
+  for (int c = 0; c < LA_RPL; ++c) acc[c] = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = part_ml[(row * nsplit + z) * 2];
+    const float lz = part_ml[(row * nsplit + z) * 2 + 1];
+    if (!(mz > -INFINITY)) continue;
+    const float w = base2 ? ldexpf(1.0f, (int)(mz - mx)) : expf(mz - mx);
+    total += lz * w;
+    const float* pa = part_acc + (row * nsplit + z) * R;
+#pragma unroll
+    for (int c = 0; c < LA_RPL; ++c) {
+      const int dd = lane + 64 * c;
+      if (dd < R) acc[c] = fmaf(pa[dd], w, acc[c]);
+    }
+  }
+  if (sink && mx > -INFINITY) {
+    const float sk = sink[row % H];
+    total += base2 ? exp2f(sk * 1.4426950408889634f - mx) : expf(sk - mx);
+  }
+  const float inv = total > 0.f ? 1.0f / total : 0.f;
+#pragma unroll
+  for (int c = 0; c < LA_RPL; ++c) {
+    const int dd = lane + 64 * c;
+    if (dd < R) out[row * R + dd] = from_f32<T>(acc[c] * inv);
+  }
+}
+
+template <typename T, int KT>
+static int launch_latent_attention(const void* q, void* out, const void* plane,
+                                   long long page_stride, const int* block_table, int bt_stride,
+                                   const int* positions, const int* wi_seq, const int* wi_row0,
+                                   const int* wi_count, int n_items, float* part_acc,
+                                   float* part_ml, int H, int HC, int W, int R, int page_size,
+                                   float scale, int keys_per_split, int nsplit, const float* sink,
+                                   hipStream_t stream) {
+  const size_t shmem = ((size_t)KT * (W + 1) + (size_t)LA_MAX_ROWS * W + LA_WAVES * 64) * sizeof(float);
+  auto kernel = latent_attention_kernel<T, KT>;
+  static size_t allowed = 0;
+  if (shmem > allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (e != hipSuccess) return (int)e;
+    allowed = shmem;
+  }
+  dim3 grid(n_items, (H + HC - 1) / HC, nsplit), block(256);
+  hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)plane,
+                     page_stride, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
+                     part_acc, part_ml, H, HC, W, R, page_size, scale, keys_per_split, nsplit, sink);
+  return za_launch_status();
+}
+
+// q: [T][H][W] folded queries; out: [T][H][R]; plane: the cache, a page's rows one after
+// the other, `page_stride` elements from page to page.  Work items: (request, first row,
+// rows), each with at most LA_MAX_ROWS / min(H, LA_MAX_ROWS) rows.
+extern "C" int za_latent_attention(const void* q, void* out, const void* plane,
+                                   long long page_stride, const int* block_table, int bt_stride,
+                                   const int* positions, const int* wi_seq, const int* wi_row0,
+                                   const int* wi_count, int n_items, int n_tokens, float* part_acc,
+                                   float* part_ml, int dtype, int heads, int width, int kv_rank,
+                                   int page_size, float scale, int keys_per_split, int nsplit,
+                                   const float* sink, hipStream_t stream) {
+  if (n_items == 0 || n_tokens == 0) return 0;
+  if (n_items < 0 || heads <= 0 || width <= 0 || kv_rank <= 0 || kv_rank > width ||
+      page_size <= 0 || bt_stride <= 0 || nsplit < 1 || !q || !out || !plane || !block_table ||
+      !positions || !wi_seq || !wi_row0 || !wi_count ||
+      page_stride < (long long)page_size * width)
+    return ZA_ERR_ARG;
+  if (width > LA_MAX_W || kv_rank > LA_MAX_R || nsplit > 65535) return ZA_ERR_UNSUPPORTED;
+  if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
+    return ZA_ERR_ARG;
+  const int HC = heads < LA_MAX_ROWS ? heads : LA_MAX_ROWS;
+  int rc;
+#define ZA_LA_ARGS                                                                             \
+  q, out, plane, page_stride, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,    \
+      n_items, part_acc, part_ml, heads, HC, width, kv_rank, page_size, scale, keys_per_split, \
+      nsplit, sink, stream
+  const bool small = width <= 256;
+  if (dtype == 0)
+    rc = small ? launch_latent_attention<float, 64>(ZA_LA_ARGS)
+               : launch_latent_attention<float, 32>(ZA_LA_ARGS);
+  else if (dtype == 1)
+    rc = small ? launch_latent_attention<bf16_t, 64>(ZA_LA_ARGS)
+               : launch_latent_attention<bf16_t, 32>(ZA_LA_ARGS);
+  else
+    return ZA_ERR_UNSUPPORTED;
+#undef ZA_LA_ARGS
+  if (rc != 0 || nsplit == 1) return rc;
+  dim3 grid((unsigned)((size_t)n_tokens * heads)), block(64);
+  if (dtype == 0)
+    hipLaunchKernelGGL((latent_combine_kernel<float>), grid, block, 0, stream, part_acc, part_ml,
+                       (float*)out, kv_rank, nsplit, 0, sink, heads);
+  else
+    hipLaunchKernelGGL((latent_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc, part_ml,
+                       (bf16_t*)out, kv_rank, nsplit, 0, sink, heads);
+  return za_launch_status();
+}

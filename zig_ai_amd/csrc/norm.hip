@@ -403,3 +403,60 @@ extern "C" int za_scaled_add_rmsnorm(float* residual, const void* a, float sa, c
 #undef ZA_SCALED_ADD
   return za_launch_status();
 }
+
+// residual += scale * y / sqrt(mean(y^2) + eps) * weight, in 32-bit, in place: something
+// that is normed by itself before it enters the stream.  A row of up to 256 * NA_VPT
+// elements stays in registers between the sum of squares and the addition.
+#define NA_VPT 16
+template <typename TD>
+__global__ void __launch_bounds__(256)
+normed_add_kernel(float* __restrict__ residual, const TD* __restrict__ y,
+                  const float* __restrict__ weight, int width, float eps, float scale) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  float* x = residual + r * width;
+  const TD* yr = y + r * width;
+  const int bd = blockDim.x;
+  float ss = 0.f;
+  if (width <= bd * NA_VPT) {
+    float v[NA_VPT];
+#pragma unroll
+    for (int k = 0; k < NA_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      v[k] = i < width ? to_f32<TD>(yr[i]) : 0.f;
+      ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, scratch);
+    const float f = scale / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int k = 0; k < NA_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      if (i < width) x[i] = fmaf(v[k] * f, weight[i], x[i]);
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < width; i += bd) {
+    const float v = to_f32<TD>(yr[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float f = scale / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += bd)
+    x[i] = fmaf(to_f32<TD>(yr[i]) * f, weight[i], x[i]);
+}
+
+extern "C" int za_normed_add(float* residual, const void* y, int y_dtype, const float* weight,
+                             int n_rows, int width, float eps, float scale, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  if (n_rows < 0 || width <= 0 || !residual || !y || !weight) return ZA_ERR_ARG;
+  dim3 grid(n_rows), block(width <= 256 ? 64 : 256);
+  if (y_dtype == 0)
+    hipLaunchKernelGGL((normed_add_kernel<float>), grid, block, 0, stream, residual,
+                       (const float*)y, weight, width, eps, scale);
+  else if (y_dtype == 1)
+    hipLaunchKernelGGL((normed_add_kernel<bf16_t>), grid, block, 0, stream, residual,
+                       (const bf16_t*)y, weight, width, eps, scale);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}

@@ -100,7 +100,7 @@ class DecoderModel:
                 note(p)
             self.blocks.append(arrangement(built, **dict(getattr(layer, "params", None) or {})))
             self.mixer_slots.append([n for n, family in slots.items() if family == "mixer"])
-        # what enters the stream between run-order entries (``LayerCall.before``)
+        # what enters the stream between run-order entries (``LayerCall.before`` / ``after``)
         self.stream_parts = [make("stream", part, ("stream", i))
                              for i, part in enumerate(getattr(spec, "stream_parts", ()))]
         for p in self.stream_parts:
@@ -254,13 +254,18 @@ class DecoderModel:
             taps.append({"stream": residual.clone()})
         # (the stream is updated in place: what may ask for the embedding's output later
         # gets a copy of it)
-        origin = residual.clone() if any(c.before is not None for c in self.schedule) else None
+        origin = residual.clone() if any(
+            getattr(self.stream_parts[c.before.part], "needs_origin", True)
+            for c in self.schedule if c.before is not None) else None
         for call, view in zip(self.schedule, views):
             step.taps = {} if taps is not None else None
             if call.before is not None:
                 residual, pending = self.stream_parts[call.before.part].forward(
                     residual, pending, origin, step, **dict(call.before.args))
             residual, pending = self.blocks[call.layer].forward(residual, pending, step, view)
+            if call.after is not None:
+                residual, pending = self.stream_parts[call.after.part].forward(
+                    residual, pending, origin, step, **dict(call.after.args))
             if taps is not None:
                 now = residual.clone()
                 if pending is not None:

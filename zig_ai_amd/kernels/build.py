@@ -28,7 +28,7 @@ PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
 SOURCES = ("norm", "gemm", "gemm_rows64", "rope_kv", "attention", "shortconv", "recurrent",
-           "activation", "experts", "sampling", "blaslt", "calibrate")
+           "activation", "experts", "latent", "sampling", "blaslt", "calibrate")
 HOST_SOURCES = ("host", "plain")    # plain C++, no device code: usable without a GPU or ROCm
 ALL_SOURCES = SOURCES + HOST_SOURCES
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]

@@ -147,6 +147,29 @@ _SIGNATURES = {
     ("experts", "za_grouped_gemm"): [c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_int, c_float, c_void_p],
+    ("activation", "za_softcap"): [c_void_p, c_float, c_longlong, c_void_p],
+    ("activation", "za_table_gate"): [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                      c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    ("norm", "za_normed_add"): [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float,
+                                c_float, c_void_p],
+    ("experts", "za_route_topk"): [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                   c_float, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    ("experts", "za_experts_combine"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                        c_int, c_void_p],
+    ("latent", "za_latent_prepare"): [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_int, c_void_p, c_void_p, c_int, c_longlong, c_int,
+                                      c_void_p],
+    ("latent", "za_rotate_part"): [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int,
+                                   c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    ("latent", "za_head_linear"): [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
+                                   c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int,
+                                   c_int, c_void_p],
+    ("latent", "za_latent_attention"): [c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                        c_float, c_int, c_int, c_void_p, c_void_p],
 }
 _functions = {}
 
@@ -2045,4 +2068,285 @@ def grouped_linear(src: torch.Tensor, weights: torch.Tensor, lists: torch.Tensor
         _ptr(counts), _ptr(out), _code(out_dtype), n_tokens, top, E, N, K, top if per_token else 1,
         1 if stacked else 0, EXPERT_ACTIVATIONS[activation], float(out_scale), _stream())
     _check(rc, "grouped_linear", f"E={E} N={N} K={K} tokens={n_tokens} top={top}")
+    return out
+
+
+def route_topk(logits: torch.Tensor, n: int, top: int, correction: Optional[torch.Tensor] = None,
+               groups: int = 0, keep: int = 0, scale: float = 1.0, scores: str = "softmax",
+               renormalize: bool = False):
+    """A router's choice: ``logits [T, >= n]`` (32-bit; the first ``n`` columns are the router's
+    outputs) -> ``(chosen [T, top] int32, weight [T, top] float32)``.  Scores are the softmax
+    over the ``n`` outputs (or ``sigmoid``); the choice goes by score plus ``correction``
+    among the outputs of the ``keep`` best of ``groups`` equal groups of neighbours (a group
+    counts by its largest choice score; ``groups = 0``: all outputs); the weight is the score
+    itself times ``scale``, with ``renormalize`` divided by the sum of the chosen scores."""
+    _need(logits, "logits", torch.float32)
+    if logits.dim() != 2 or logits.shape[1] < n:
+        raise KernelError(f"logits must be [T, >= {n}], got {tuple(logits.shape)}")
+    if scores not in ("softmax", "sigmoid"):
+        raise KernelError(f"scores must be softmax or sigmoid, got {scores!r}")
+    T = logits.shape[0]
+    if correction is not None:
+        _need(correction, "correction", torch.float32, (n,))
+    chosen = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    rc = _fn("experts", "za_route_topk")(
+        _ptr(logits), logits.shape[1], _ptr(correction), T, int(n), int(groups), int(keep),
+        int(top), float(scale), 0 if scores == "softmax" else 1, 1 if renormalize else 0,
+        _ptr(chosen), _ptr(weight), _stream())
+    _check(rc, "route_topk", f"n={n} top={top} groups={groups} keep={keep}")
+    return chosen, weight
+
+
+def experts_combine(expert_out: Optional[torch.Tensor], chosen: torch.Tensor, weight: torch.Tensor,
+                    x: torch.Tensor, n_real: int, shared: Optional[torch.Tensor] = None,
+                    gate_logits: Optional[torch.Tensor] = None, gate_col: int = 0) -> torch.Tensor:
+    """``y[t] = sum_j weight[t, j] * (expert_out[t * top + j] if chosen[t, j] < n_real else
+    x[t]) + gate(t) * shared[t]`` as 32-bit ``[T, width]``; ``gate(t)`` is
+    ``sigmoid(gate_logits[t, gate_col])`` (32-bit logits) or one."""
+    T, top = chosen.shape
+    _need(chosen, "chosen", torch.int32, (T, top))
+    _need(weight, "weight", torch.float32, (T, top))
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    width = x.shape[1]
+    dtype = None
+    if expert_out is not None:
+        _need(expert_out, "expert_out", (torch.float32, torch.bfloat16), (T * top, width))
+        dtype = expert_out.dtype
+    elif n_real > 0:
+        raise KernelError("experts with weights need their outputs")
+    if shared is not None:
+        _need(shared, "shared", dtype or (torch.float32, torch.bfloat16), (T, width))
+        dtype = shared.dtype
+    gate_ld = 0
+    gate_ptr = None
+    if gate_logits is not None:
+        _need(gate_logits, "gate_logits", torch.float32)
+        if gate_logits.dim() != 2 or gate_logits.shape[0] != T or not 0 <= gate_col < gate_logits.shape[1]:
+            raise KernelError(f"gate_logits has shape {tuple(gate_logits.shape)}; column {gate_col} "
+                              f"of {T} rows is needed")
+        gate_ld = gate_logits.shape[1]
+        gate_ptr = gate_logits.data_ptr() + 4 * gate_col
+    y = torch.empty((T, width), dtype=torch.float32, device=x.device)
+    rc = _fn("experts", "za_experts_combine")(
+        _ptr(expert_out), _code(dtype or torch.float32), _ptr(chosen), _ptr(weight), _ptr(x),
+        _code(x.dtype), _ptr(shared), gate_ptr, gate_ld, _ptr(y), T, top, int(n_real), width,
+        _stream())
+    _check(rc, "experts_combine")
+    return y
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` for a 32-bit tensor, in place."""
+    _need(x, "x", torch.float32)
+    rc = _fn("activation", "za_softcap")(_ptr(x), float(cap), x.numel(), _stream())
+    _check(rc, "softcap_")
+    return x
+
+
+def table_gate(g: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int,
+               activation: str) -> torch.Tensor:
+    """``act(g[t, j]) * table[ids[t], col0 + j]`` for ``g [T, dim]``: a gate on a slice of the
+    table row that each token's id picks; ``activation`` as for ``gated_unit``."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"activation must be one of {sorted(GATE_ACTIVATIONS)}, got {activation!r}")
+    _need(g, "g", (torch.float32, torch.bfloat16))
+    if g.dim() != 2:
+        raise KernelError(f"table_gate takes [T, dim], got {tuple(g.shape)}")
+    T, dim = g.shape
+    _need(ids, "ids", torch.int32, (T,))
+    _need(table, "table", (torch.float32, torch.bfloat16))
+    if table.dim() != 2 or col0 < 0 or col0 + dim > table.shape[1]:
+        raise KernelError(f"columns [{col0}, {col0 + dim}) of a table {tuple(table.shape)}")
+    out = torch.empty_like(g)
+    rc = _fn("activation", "za_table_gate")(
+        _ptr(g), _code(g.dtype), _ptr(ids), _ptr(table), _code(table.dtype), table.shape[0],
+        table.shape[1], int(col0), _ptr(out), T, dim, GATE_ACTIVATIONS[activation], _stream())
+    _check(rc, "table_gate")
+    return out
+
+
+def normed_add_(stream: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+                scale: float = 1.0) -> torch.Tensor:
+    """``stream += scale * y / sqrt(mean(y^2) + eps) * weight`` in 32-bit, in place."""
+    n, width = stream.shape
+    _need(stream, "stream", torch.float32, (n, width))
+    _need(y, "y", (torch.float32, torch.bfloat16), (n, width))
+    _need(weight, "weight", torch.float32, (width,))
+    rc = _fn("norm", "za_normed_add")(_ptr(stream), _ptr(y), _code(y.dtype), _ptr(weight), n, width,
+                                      float(eps), float(scale), _stream())
+    _check(rc, "normed_add_")
+    return stream
+
+
+# ------------------------------------------------------------ latent attention
+LATENT_MAX_ROWS = 32        # rows (token, head) of a work item of the general kernel
+LATENT_MAX_WIDTH = 576      # cached elements a token
+LATENT_MAX_RANK = 512       # of which the latent
+
+
+def _latent_plane(plane: torch.Tensor, dtype, width: int) -> Tuple[int, int]:
+    """The cache of one layer as the latent kernels index it: ``[pages, 1, page_size, width]``,
+    the rows of a page one after the other.  Returns (page size, elements from page to page)."""
+    if not isinstance(plane, torch.Tensor) or not plane.is_cuda or plane.dtype != dtype:
+        raise KernelError(f"the latent cache must be a GPU tensor of {dtype}")
+    if plane.dim() != 4 or plane.shape[1] != 1 or plane.shape[3] != width \
+            or plane.stride()[1:] != (plane.shape[2] * width, width, 1) \
+            or plane.stride(0) < plane.shape[2] * width:
+        raise KernelError(f"the latent cache has shape {tuple(plane.shape)} and strides "
+                          f"{plane.stride()}, expected [pages, 1, page_size, {width}]")
+    return plane.shape[2], plane.stride(0)
+
+
+def latent_prepare(down: torch.Tensor, q_col: int, q_rank: int, c_col: int, kv_rank: int,
+                   rot_dim: int, q_norm_w: torch.Tensor, c_norm_w: torch.Tensor, eps: float,
+                   positions: torch.Tensor, slots: Optional[torch.Tensor],
+                   inv_freq: Optional[torch.Tensor], rot_dims: int, adjacent_pairs: bool,
+                   plane: Optional[torch.Tensor]) -> torch.Tensor:
+    """From the rows of a latent attention's opening projection ``down [T, columns]``: the
+    RMS-normed query latent ``[T, q_rank]`` (returned), and, with ``plane``, each token's
+    cached row ``[rmsnorm(latent) | rotated key part]`` written to its place ``slots[t]``."""
+    _need(down, "down", (torch.float32, torch.bfloat16))
+    T, ld = down.shape
+    _need(q_norm_w, "q_norm_w", torch.float32, (q_rank,))
+    _need(c_norm_w, "c_norm_w", torch.float32, (kv_rank,))
+    _need(positions, "positions", torch.int32, (T,))
+    if q_col < 0 or q_col + q_rank > ld or c_col < 0 or c_col + kv_rank + rot_dim > ld:
+        raise KernelError(f"the projection's rows hold {ld} elements")
+    if rot_dims % 2 or not 0 <= rot_dims <= rot_dim:
+        raise KernelError(f"rot_dims {rot_dims} must be even and at most {rot_dim}")
+    if rot_dims:
+        _need(inv_freq, "inv_freq", torch.float32, (rot_dims // 2,))
+    page_size = stride = 0
+    if plane is not None:
+        _need(slots, "slots", torch.int32, (T,))
+        page_size, stride = _latent_plane(plane, down.dtype, kv_rank + rot_dim)
+    cq = torch.empty((T, q_rank), dtype=down.dtype, device=down.device)
+    rc = _fn("latent", "za_latent_prepare")(
+        _ptr(down), _code(down.dtype), ld, int(q_col), int(q_rank), int(c_col), int(kv_rank),
+        int(rot_dim), _ptr(q_norm_w), _ptr(c_norm_w), float(eps), _ptr(positions),
+        _ptr(slots) if plane is not None else None, _ptr(inv_freq) if rot_dims else None,
+        int(rot_dims), 1 if adjacent_pairs else 0, _ptr(cq), _ptr(plane), page_size, stride, T,
+        _stream())
+    _check(rc, "latent_prepare")
+    return cq
+
+
+def rotate_part_(src: torch.Tensor, src_col: int, dst: torch.Tensor, dst_col: int, rot_dim: int,
+                 positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot_dims: int,
+                 adjacent_pairs: bool) -> torch.Tensor:
+    """``dst[t, h, dst_col : dst_col + rot_dim]`` takes ``src[t, h, src_col : ...]`` with its
+    first ``rot_dims`` elements rotated by the token's position."""
+    _need(src, "src", (torch.float32, torch.bfloat16))
+    _need(dst, "dst", src.dtype)
+    if src.dim() != 3 or dst.dim() != 3 or src.shape[:2] != dst.shape[:2]:
+        raise KernelError(f"rotate_part_ takes [T, heads, width] tensors, got {tuple(src.shape)} "
+                          f"and {tuple(dst.shape)}")
+    T, H = src.shape[:2]
+    if src_col < 0 or src_col + rot_dim > src.shape[2] or dst_col < 0 \
+            or dst_col + rot_dim > dst.shape[2]:
+        raise KernelError("the rotated part does not fit the rows")
+    _need(positions, "positions", torch.int32, (T,))
+    if rot_dims:
+        _need(inv_freq, "inv_freq", torch.float32, (rot_dims // 2,))
+    rc = _fn("latent", "za_rotate_part")(
+        _ptr(src), _code(src.dtype), src.shape[2], int(src_col), _ptr(dst), dst.shape[2],
+        int(dst_col), T, H, int(rot_dim), _ptr(positions), _ptr(inv_freq) if rot_dims else None,
+        int(rot_dims), 1 if adjacent_pairs else 0, _stream())
+    _check(rc, "rotate_part_")
+    return dst
+
+
+HEAD_GATES = {None: 0, "head": 1, "element": 2}
+
+
+def head_linear(x: torch.Tensor, x_col: int, weight: torch.Tensor, out: Optional[torch.Tensor] = None,
+                out_col: int = 0, out_dtype: Optional[torch.dtype] = None,
+                gate: Optional[torch.Tensor] = None, gate_col: int = 0,
+                gate_mode: Optional[str] = None) -> torch.Tensor:
+    """Every head's own product at once: ``out[t, h, out_col + n] = sum_k x[t, h, x_col + k] *
+    weight[h, n, k]`` for ``x [T, heads, any width]`` and ``weight [heads, N, K]``; ``out`` is
+    ``[T, heads, >= out_col + N]`` (a new ``[T, heads, N]`` if not given).  With ``gate [T,
+    columns]`` (pre-sigmoid, of ``x``'s type) the result is multiplied by ``sigmoid(gate[t,
+    gate_col + h])`` (``gate_mode="head"``) or ``sigmoid(gate[t, gate_col + h * N + n])``
+    (``"element"``).  bfloat16 weights run on the matrix cores, 32-bit weights the FMA form
+    (with ``x`` of either type)."""
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    _need(weight, "weight", (torch.float32, torch.bfloat16))
+    if x.dim() != 3 or weight.dim() != 3 or weight.shape[0] != x.shape[1]:
+        raise KernelError(f"head_linear takes x [T, heads, width] and weight [heads, N, K], got "
+                          f"{tuple(x.shape)} and {tuple(weight.shape)}")
+    T, H, x_ld = x.shape
+    _, N, K = weight.shape
+    if x_col < 0 or x_col + K > x_ld:
+        raise KernelError(f"columns [{x_col}, {x_col + K}) of rows of {x_ld}")
+    if weight.dtype == torch.bfloat16 and (x.dtype != torch.bfloat16 or K % 8 or x_ld % 8 or x_col % 8):
+        raise KernelError("bfloat16 head weights need bfloat16 rows whose pieces start on 16-byte "
+                          "boundaries; keep the weight in 32-bit otherwise")
+    if gate_mode not in HEAD_GATES:
+        raise KernelError(f"gate_mode must be None, head or element, got {gate_mode!r}")
+    if out is None:
+        out = torch.empty((T, H, N), dtype=out_dtype or x.dtype, device=x.device)
+        out_col = 0
+    _need(out, "out", (torch.float32, torch.bfloat16))
+    if out.dim() != 3 or tuple(out.shape[:2]) != (T, H) or out_col < 0 or out_col + N > out.shape[2]:
+        raise KernelError(f"out has shape {tuple(out.shape)}")
+    gate_ld = 0
+    if gate_mode is not None:
+        _need(gate, "gate", x.dtype)
+        need = H if gate_mode == "head" else H * N
+        if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + need > gate.shape[1]:
+            raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
+                              f"{gate_col + need} of {T} rows are needed")
+        gate_ld = gate.shape[1]
+    rc = _fn("latent", "za_head_linear")(
+        _ptr(x), _code(x.dtype), x_ld, int(x_col), _ptr(weight), _code(weight.dtype), _ptr(out),
+        _code(out.dtype), out.shape[2], int(out_col), T, H, N, K,
+        _ptr(gate) if gate_mode is not None else None, gate_ld, int(gate_col),
+        HEAD_GATES[gate_mode], _stream())
+    _check(rc, "head_linear", f"T={T} H={H} N={N} K={K}")
+    return out
+
+
+def latent_attention(q: torch.Tensor, plane: torch.Tensor, kv_rank: int, block_table: torch.Tensor,
+                     positions: torch.Tensor, item_seq: torch.Tensor, item_row0: torch.Tensor,
+                     item_count: torch.Tensor, n_items: int, scale: float,
+                     sink: Optional[torch.Tensor] = None, keys_per_split: int = 0,
+                     nsplit: int = 1) -> torch.Tensor:
+    """Causal attention of the folded queries ``q [T, heads, width]`` over cached rows of
+    ``width`` elements whose first ``kv_rank`` are also the values; returns ``[T, heads,
+    kv_rank]``.  ``item_*``: work items of at most ``LATENT_MAX_ROWS // min(heads,
+    LATENT_MAX_ROWS)`` consecutive rows of one request.  ``sink``: 32-bit ``[heads]``."""
+    if q.dim() != 3:
+        raise KernelError(f"q must be [T, heads, width], got {tuple(q.shape)}")
+    T, H, W = q.shape
+    _need(q, "q", (torch.float32, torch.bfloat16))
+    page_size, stride = _latent_plane(plane, q.dtype, W)
+    if not 0 < kv_rank <= W or W > LATENT_MAX_WIDTH or kv_rank > LATENT_MAX_RANK:
+        raise KernelError(f"a latent of {kv_rank} in rows of {W}: the kernel takes rows up to "
+                          f"{LATENT_MAX_WIDTH} and latents up to {LATENT_MAX_RANK}")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [requests, max_pages]")
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    if sink is not None:
+        _need(sink, "sink", torch.float32, (H,))
+    out = torch.empty((T, H, kv_rank), dtype=q.dtype, device=q.device)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        part_acc = torch.empty((T, H, nsplit, kv_rank), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, H, nsplit, 2), dtype=torch.float32, device=q.device)
+    rc = _fn("latent", "za_latent_attention")(
+        _ptr(q), _ptr(out), _ptr(plane), stride, _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+        _ptr(part_acc), _ptr(part_ml), _code(q.dtype), H, W, int(kv_rank), page_size, float(scale),
+        int(keys_per_split), int(nsplit), _ptr(sink), _stream())
+    _check(rc, "latent_attention")
+    _note("attention", kernel="latent", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out

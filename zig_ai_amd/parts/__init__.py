@@ -5,5 +5,5 @@ from .base import (FeedForward, Mixer, Norm, PagedNeed, Part, PositionEncoding, 
                    StateNeed, TensorRule, lookup, register_arrangement, register_embedding,
                    register_feed_forward, register_head, register_mixer, register_norm,
                    register_position)
-from . import (norm, rope, feed_forward, experts, embedding, attention, short_conv, recurrent,  # noqa: F401
-               block, stream)
+from . import (norm, rope, feed_forward, experts, embedding, attention, latent_attention,  # noqa: F401
+               short_conv, recurrent, block, stream)

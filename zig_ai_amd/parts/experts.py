@@ -80,3 +80,117 @@ class TableExperts(FeedForward):
 
 
 register_feed_forward(TableExperts.kind, TableExperts)
+
+
+class RoutedExperts(FeedForward):
+    """Small gated experts of which a router picks ``top`` for every token:
+
+        z = Wr x;  s = softmax(z) over all router outputs  (``scores="sigmoid"``: sigmoid(z))
+        the choice goes by s + correction (``correction``: a tensor, used for the choice
+        only), among the outputs of the ``groups_kept`` best of ``groups`` equal groups of
+        neighbouring outputs (a group counts by its largest choice score; ``groups = 0``: no
+        limit); weight = s * route_scale (``renormalize``: divided by the chosen scores' sum)
+        y = sum_chosen weight_e * expert_e(x) + gate * shared(x)
+
+    ``expert_e(x) = Wdown_e (act(Wgate_e x) * (Wup_e x))`` for the ``experts`` outputs that have
+    weights; the ``identity_experts`` outputs behind them hand ``x`` on.  ``shared_size > 0``:
+    one more expert of that width runs for every token, times ``sigmoid(Wsg x)`` (one number
+    a token) when ``shared_gate``.  The router's product and everything after it up to the
+    weights is 32-bit; the weighted sum is taken in 32-bit in a fixed order.
+
+    Nothing is looked at on the host: the router's choice becomes per-expert lists on the
+    device and two grouped products run every expert's rows in one launch each."""
+
+    kind = "routed_experts"
+    graph_safe = True
+    kernel_sources = ("experts", "gemm", "gemm_rows64", "activation")
+
+    @staticmethod
+    def _sizes(params):
+        return (int(params["hidden_size"]), int(params.get("intermediate_size") or 0),
+                int(params["experts"]), int(params.get("identity_experts") or 0),
+                int(params["top"]), int(params.get("shared_size") or 0))
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, I, E, ident, top, S = cls._sizes(params)
+        rules = {"router.weight": TensorRule(((E + ident, H),))}
+        if params.get("correction"):
+            rules["correction"] = TensorRule(((E + ident,),), role="bias")
+        for e in range(E):
+            rules[f"experts.{e}.gate.weight"] = TensorRule(((I, H),))
+            rules[f"experts.{e}.up.weight"] = TensorRule(((I, H),))
+            rules[f"experts.{e}.down.weight"] = TensorRule(((H, I),))
+        if S:
+            rules["shared.gate.weight"] = TensorRule(((S, H),))
+            rules["shared.up.weight"] = TensorRule(((S, H),))
+            rules["shared.down.weight"] = TensorRule(((H, S),))
+            if params.get("shared_gate"):
+                rules["shared.token_gate.weight"] = TensorRule(((1, H),))
+        return rules
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        H, I, E, ident, top, S = self._sizes(params)
+        n = E + ident
+        if not 0 < top <= n or n > ops.EXPERTS_MAX:
+            raise ValueError(f"{top} of {n} router outputs: top must be within 1..outputs, outputs "
+                             f"at most {ops.EXPERTS_MAX}")
+        self.experts, self.identity, self.top, self.outputs = E, ident, top, n
+        self.groups = int(params.get("groups") or 0)
+        self.keep = int(params.get("groups_kept") or 0)
+        if self.groups and (n % self.groups or not 0 < self.keep <= self.groups
+                            or self.keep * (n // self.groups) < top):
+            raise ValueError(f"{n} router outputs in {self.groups} groups of which {self.keep} are "
+                             f"kept cannot yield {top}")
+        self.route_scale = float(params.get("route_scale", 1.0))
+        self.scores = str(params.get("scores", "softmax"))
+        self.renormalize = bool(params.get("renormalize", False))
+        self.activation = str(params.get("activation", "silu"))
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"expert activation must be one of {sorted(ops.GATE_ACTIVATIONS)}, "
+                             f"got {self.activation!r}")
+        self.correction = tensors["correction"] if params.get("correction") else None
+        # the router's rows and, behind them, the shared expert's gate: one 32-bit product
+        rows = [tensors["router.weight"]]
+        self.shared_gated = bool(S and params.get("shared_gate"))
+        if self.shared_gated:
+            rows.append(tensors["shared.token_gate.weight"])
+        self.w_router = ops.projection_weight(torch.cat(rows, dim=0).contiguous())
+        self.gate_up = self.down = None
+        if E:
+            self.gate_up = TableExperts._stack(
+                [torch.cat([tensors[f"experts.{e}.gate.weight"], tensors[f"experts.{e}.up.weight"]],
+                           dim=0) for e in range(E)])
+            self.down = TableExperts._stack([tensors[f"experts.{e}.down.weight"] for e in range(E)])
+        self.shared_gate_up = self.shared_down = None
+        if S:
+            self.shared_gate_up = ops.projection_weight(
+                torch.cat([tensors["shared.gate.weight"], tensors["shared.up.weight"]], dim=0).contiguous())
+            self.shared_down = ops.projection_weight(tensors["shared.down.weight"])
+
+    def forward(self, x, step):
+        T = x.shape[0]
+        tune = self.runtime.tune
+        logits = ops.linear(x, self.w_router, out_dtype=torch.float32, tune=tune)
+        chosen, weight = ops.route_topk(logits, self.outputs, self.top, self.correction,
+                                        self.groups, self.keep, self.route_scale, self.scores,
+                                        self.renormalize)
+        out = None
+        if self.experts:
+            # an output beyond the experts that have weights is in nobody's list
+            lists, counts = ops.expert_lists(None, chosen, T, self.experts)
+            a = ops.grouped_linear(x, self.gate_up, lists, counts, T, per_token=True,
+                                   out_dtype=x.dtype)
+            a = ops.gated_unit(a, self.activation)
+            out = ops.grouped_linear(a, self.down, lists, counts, T, per_token=False,
+                                     out_dtype=torch.float32)
+        shared = None
+        if self.shared_gate_up is not None:
+            s = ops.gated_unit(ops.linear(x, self.shared_gate_up, tune=tune), self.activation)
+            shared = ops.linear(s, self.shared_down, out_dtype=torch.float32, tune=tune)
+        return ops.experts_combine(out, chosen, weight, x, self.experts, shared,
+                                   logits if self.shared_gated else None, self.outputs)
+
+
+register_feed_forward(RoutedExperts.kind, RoutedExperts)

@@ -45,3 +45,65 @@ class PassOffset(Part):
 
 
 register_stream_step(PassOffset.kind, PassOffset)
+
+
+class TokenSide(Part):
+    """What a layer takes from the tokens themselves, past its mixer and feed-forward
+    (``token_side``).  A second embedding table ``[vocab, layers * dim]`` holds ``dim`` numbers
+    for every layer and token id; for layer ``i``
+
+        e = table[token, i * dim : (i + 1) * dim]
+        g = act(Wgate_i x) * e                 x: the stream itself, not normed
+        y = Wproj_i g
+        x <- x (+ pending) + scale * y / sqrt(mean(y^2) + eps) * norm_i
+
+    ``layers``, ``dim``, ``width``, ``vocab_size``, ``eps``, ``scale`` and ``activation`` are
+    parameters; a run-order entry names the layer with ``args = {"layer": i}``."""
+
+    kind = "token_side"
+    graph_safe = True
+    needs_origin = False
+    kernel_sources = ("norm", "gemm", "gemm_rows64", "activation")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        L, dim, width = int(params["layers"]), int(params["dim"]), int(params["width"])
+        rules = {"table": TensorRule(((int(params["vocab_size"]), L * dim),), role="table")}
+        for i in range(L):
+            rules[f"layers.{i}.gate.weight"] = TensorRule(((dim, width),))
+            rules[f"layers.{i}.proj.weight"] = TensorRule(((width, dim),))
+            rules[f"layers.{i}.norm.weight"] = TensorRule(((width,),), role="norm")
+        return rules
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.layers, self.dim = int(params["layers"]), int(params["dim"])
+        self.eps = float(params["eps"])
+        self.scale = float(params.get("scale", 1.0))
+        self.activation = str(params.get("activation", "gelu_tanh"))
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"activation must be one of {sorted(ops.GATE_ACTIVATIONS)}, got "
+                             f"{self.activation!r}")
+        self.table = tensors["table"]
+        self.gate = [ops.projection_weight(tensors[f"layers.{i}.gate.weight"])
+                     for i in range(self.layers)]
+        self.proj = [ops.projection_weight(tensors[f"layers.{i}.proj.weight"])
+                     for i in range(self.layers)]
+        self.norm = [tensors[f"layers.{i}.norm.weight"] for i in range(self.layers)]
+
+    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor],
+                origin: Optional[torch.Tensor], step, layer: int = 0):
+        i = int(layer)
+        if not 0 <= i < self.layers:
+            raise ValueError(f"layer {layer} of {self.layers}")
+        if pending is not None:
+            ops.stream_add_(residual, pending)
+        x = ops.cast(residual, self.runtime.dtype)
+        g = ops.table_gate(ops.linear(x, self.gate[i], tune=self.runtime.tune), step.token_ids,
+                           self.table, i * self.dim, self.activation)
+        y = ops.linear(g, self.proj[i], out_dtype=torch.float32, tune=self.runtime.tune)
+        ops.normed_add_(residual, y, self.norm[i], self.eps, self.scale)
+        return residual, None
+
+
+register_stream_step(TokenSide.kind, TokenSide)
