@@ -64,10 +64,13 @@ def sink_softmax(s: torch.Tensor, sink: torch.Tensor) -> torch.Tensor:
 
 # ------------------------------------------------------------- latent attention
 def latent_attention(h: torch.Tensor, tensors, p: str, m: Mapping, eps: float,
-                     rotated: bool, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     rotated: bool, positions: Optional[torch.Tensor] = None,
+                     reach: int = 0) -> torch.Tensor:
     """Queries through a normed latent; keys and values of every head expanded from one
     normed latent a token; with ``rotated`` a rotated key part shared by all heads beside
-    each head's unrotated one, and a gate an element; without, a gate a head."""
+    each head's unrotated one, and a gate an element; without, a gate a head.  ``reach``
+    is 0; tests that ask whether a mask that is one token off would show set it to -1 (a
+    query does not see itself) or 1 (it sees its successor)."""
     T = h.shape[0]
     H, d, dv, r = int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"])
     dr = int(m["rot_dim"]) if rotated else 0
@@ -84,7 +87,7 @@ def latent_attention(h: torch.Tensor, tensors, p: str, m: Mapping, eps: float,
         q_rot = rotate_pairs(q_rot, pos, int(rot["dims"]), float(rot["base"]))
         k_rot = rotate_pairs(down[:, r:r + dr], pos, int(rot["dims"]), float(rot["base"]))
     sink = _w(tensors, p + "sink")
-    causal = pos[None, :] <= pos[:, None]
+    causal = pos[None, :] <= pos[:, None] + reach
     out = torch.zeros((T, H, dv), dtype=DT)
     for hh in range(H):
         s = q_plain[:, hh] @ k[:, hh].T
