@@ -5,6 +5,7 @@
     python bench.py --shape 350m --workload serve         # 64 requests through the scheduler
     python bench.py --workload compare                    # Rudilix beside LFM2 at equal sizes
     python bench.py --workload compare --compare-design ranesun   # Ranesun beside Rudilix
+    python bench.py --workload compare --compare-design gemodra   # Gemodra beside Ranesun
 
 Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
@@ -36,6 +37,10 @@ width (``--compare-widths``), as one JSON line.  ``--compare-design ranesun``: a
 (retention and sink attention layers in turn, dense and table-routed feed-forwards in turn,
 the first half of the layers as a looped span) beside a Rudilix model of the same width,
 depth and vocabulary, the closest design the engine has (recurrent and attention layers).
+``--compare-design gemodra``: a Gemodra model (attention over a cached latent in every layer,
+every fourth without positions; routed small experts with a shared one; a token input a
+layer) beside a Ranesun model of the same width, depth and vocabulary, the closest design
+the engine has (attention with sinks, experts of which a token uses a few).
 """
 
 import argparse
@@ -184,9 +189,34 @@ def ranesun_shape(width, layers, vocab):
             "layers": out, "max_position_embeddings": 128000}
 
 
+def gemodra_shape(width, layers, vocab):
+    """Layer sizes in the manner of a real model of this design: heads of 128 unrotated and 64
+    rotated elements with values of 128 over a latent of 512 (queries through a latent of
+    three quarters of the width), every fourth layer the form without positions; 30 experts of
+    half the width and 2 identity outputs in 4 groups of which 2 are kept, 4 a token, beside a
+    shared expert of the width; a token input of 256 numbers a layer."""
+    heads = width // 128
+    rotated = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+               "q_rank": 3 * width // 4, "scale": 192 ** -0.5, "rot": {"dims": 64, "base": 1e6}}
+    plain = {"heads": heads, "dim": 128, "vdim": 128, "kv_rank": 512, "q_rank": 3 * width // 4,
+             "scale": 128 ** -0.5}
+    mlp = {"kind": "moe", "expert": {"ff": width // 2}, "shared": {"ff": width},
+           "router": {"experts": 30, "identity": 2, "top": 4, "scale": 2.0,
+                      "groups": {"count": 4, "keep": 2}}}
+    out = []
+    for i in range(layers):
+        kind = "latent_attention_2" if i % 4 == 3 else "latent_attention"
+        out.append({"type": kind, "mixer": plain if kind == "latent_attention_2" else rotated,
+                    "mlp": mlp})
+    return {"architecture": "Gemodra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "residual_mult": 0.5, "logit_softcap": 30.0, "token_side": {"dim": 256},
+            "layers": out, "max_position_embeddings": 128000}
+
+
 def compare(widths, layers, batch, prompt_len, steps, warmup, design="rudilix", only=None) -> dict:
     """Prefill and decode throughput of Rudilix and of LFM2 at equal sizes, or
-    (``design="ranesun"``) of Ranesun and of Rudilix."""
+    (``design="ranesun"``) of Ranesun and of Rudilix, or (``design="gemodra"``) of Gemodra and
+    of Ranesun."""
     import torch
     from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
     from zig_ai_amd.kernels import ops
@@ -275,9 +305,10 @@ def compare(widths, layers, batch, prompt_len, steps, warmup, design="rudilix", 
 
     result = {"workload": "compare", "dtype": "bf16", "data": "synthetic", "layers": layers,
               "batch": batch, "prompt_len": prompt_len, "steps": steps, "warmup": warmup, "widths": {}}
-    if design == "ranesun":
+    if design in ("ranesun", "gemodra"):
         for width in widths:
-            pair = {"ranesun": ranesun_shape, "rudilix": rudilix_shape}
+            pair = {"ranesun": ranesun_shape, "rudilix": rudilix_shape} if design == "ranesun" \
+                else {"gemodra": gemodra_shape, "ranesun": ranesun_shape}
             result["widths"][str(width)] = {name: measure(shape(width, layers, vocab))
                                             for name, shape in pair.items()
                                             if only in (None, name)}
@@ -337,8 +368,9 @@ def main() -> int:
     ap.add_argument("--compare-widths", default="1024,2048",
                     help="--workload compare: the widths, with commas between them")
     ap.add_argument("--compare-layers", type=int, default=8, help="--workload compare: layers")
-    ap.add_argument("--compare-design", choices=["rudilix", "ranesun"], default="rudilix",
-                    help="--workload compare: rudilix (beside LFM2) or ranesun (beside Rudilix)")
+    ap.add_argument("--compare-design", choices=["rudilix", "ranesun", "gemodra"], default="rudilix",
+                    help="--workload compare: rudilix (beside LFM2), ranesun (beside Rudilix) or "
+                         "gemodra (beside Ranesun)")
     ap.add_argument("--compare-only", default=None,
                     help="--workload compare: measure this model of the pair alone (for a profiler)")
     ap.add_argument("--workload", choices=["steps", "serve", "compare"], default="steps",

@@ -534,6 +534,75 @@ def test_router_kernel(n, top, groups, scale):
                 assert abs(got[(t, e)] - w) < 1e-6 + 1e-5 * abs(w)
 
 
+def _latent_attention_case(dtype, H, W, R, requests, page_size, per_item, seed):
+    """A paged cache of rows ``[latent | rotated part]`` for ``requests`` = [(cached, new)],
+    folded queries for the new tokens, the step's arrays, and what the attention should give
+    (float64, with a sink a head)."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum(-(-(c + n) // page_size) for c, n in requests) + 3
+    order = torch.randperm(n_pages, generator=g).tolist()
+    plane = torch.zeros(n_pages, 1, page_size, W)
+    most = max(-(-(c + n) // page_size) for c, n in requests)
+    table = torch.full((len(requests), most + 1), -1, dtype=torch.int32)
+    scale = 1.7 * W ** -0.5
+    sink = torch.randn(H, generator=g) * 1.5
+    qs, positions, items, want = [], [], [], []
+    row = 0
+    for s, (cached, new) in enumerate(requests):
+        keys = (torch.randn(cached + new, W, generator=g)).to(dtype).float()
+        for p in range(-(-(cached + new) // page_size)):
+            page = order.pop()
+            table[s, p] = page
+            chunk = keys[p * page_size:(p + 1) * page_size]
+            plane[page, 0, :chunk.shape[0]] = chunk
+        q = torch.randn(new, H, W, generator=g).to(dtype).float()
+        qs.append(q)
+        positions += list(range(cached, cached + new))
+        for a in range(0, new, per_item):
+            items.append((s, row + a, min(per_item, new - a)))
+        row += new
+        for i in range(new):
+            k = keys[:cached + i + 1].double()
+            sc = torch.einsum("hw,jw->hj", q[i].double(), k) * scale
+            top = torch.maximum(sc.max(dim=1, keepdim=True).values, sink.double()[:, None])
+            e = torch.exp(sc - top)
+            pr = e / (e.sum(dim=1, keepdim=True) + torch.exp(sink.double()[:, None] - top))
+            want.append(pr @ k[:, :R])
+    dev = torch.device("cuda")
+    mk = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    return (torch.cat(qs).to(dtype).to(dev), plane.to(dtype).to(dev), table.to(dev), mk(positions),
+            mk([i[0] for i in items]), mk([i[1] for i in items]), mk([i[2] for i in items]),
+            len(items), scale, sink.to(dev), torch.stack(want))
+
+
+@pytest.mark.parametrize("H,W,R,page_size", [(3, 40, 32, 4), (16, 576, 512, 16), (8, 160, 128, 16),
+                                             (4, 96, 96, 16), (5, 48, 24, 8), (40, 80, 72, 16),
+                                             (1, 264, 256, 32)])
+def test_latent_attention_kernels(H, W, R, page_size):
+    from zig_ai_amd.kernels import ops
+    # prompt portions behind cached tokens, a first portion, single tokens, one token alone
+    requests = [(70, 9), (0, 45), (133, 1), (0, 1), (31, 2)]
+    for dtype, waves_list in ((torch.float32, (0,)), (torch.bfloat16, (0, 4))):
+        for waves in waves_list:
+            most = ops.LATENT_MFMA_ROWS if waves else ops.LATENT_MAX_ROWS
+            per_item = max(1, most // min(H, most))
+            q, plane, table, pos, iseq, irow, icnt, n, scale, sink, want = _latent_attention_case(
+                dtype, H, W, R, requests, page_size, per_item, seed=H + W)
+            for keys, nsplit in ((0, 1), (64, 3)):
+                got = ops.latent_attention(q, plane, R, table, pos, iseq, irow, icnt, n, scale, sink,
+                                           keys, nsplit, waves).cpu().double()
+                tol = 2e-5 if dtype == torch.float32 else 2e-2
+                assert float((got - want).abs().max()) < tol, (dtype, waves, nsplit)
+    # single tokens only: a wave a workgroup
+    requests = [(200, 1), (0, 1), (63, 1), (64, 1)]
+    q, plane, table, pos, iseq, irow, icnt, n, scale, sink, want = _latent_attention_case(
+        torch.bfloat16, H, W, R, requests, page_size, 1, seed=7)
+    for keys, nsplit in ((0, 1), (64, 4), (128, 2)):
+        got = ops.latent_attention(q, plane, R, table, pos, iseq, irow, icnt, n, scale, sink, keys,
+                                   nsplit, 1).cpu().double()
+        assert float((got - want).abs().max()) < 2e-2, nsplit
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,N,K,mode", [(3, 24, 16, None), (8, 128, 64, "element"), (5, 40, 32, "head"),
                                         (1, 8, 320, "element"), (40, 72, 8, None)])

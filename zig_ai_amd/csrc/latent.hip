@@ -500,6 +500,217 @@ latent_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* _
   }
 }
 
+// ------------------------------------------------------------ latent_attention_mfma
+// bfloat16 on the matrix cores, rows of W and latents of R elements that are multiples of 8
+// (16-byte pieces).  A workgroup of NW waves serves one work item and one chunk of heads,
+// at most NW * 16 rows (token, head); each wave owns 16 of them.  Per tile of 32 keys:
+//   staging  every thread fetches, for 8 keys, the same 8 latent elements (eight 16-byte
+//            loads), stores them as they are into Ks [32][W] and, turned round in its
+//            registers, into Vt [R][32]: the second product wants, for one latent element,
+//            consecutive keys side by side.  The rotated key part goes into Ks only.
+//   S^T = K Q^T   keys are the rows of the first operand, the wave's 16 query rows the
+//            columns: a lane ends up with ONE query row's scores for keys kq*4 .. +3 of
+//            each half of the tile (kq = lane / 16)
+//   p = 2^(s * scale * log2(e) - m) in 32-bit, the running maximum shared by the four lanes
+//            of a query row; p is rounded to bfloat16 and the sum that normalises the result
+//            is the sum of the rounded values
+//   O^T += V^T P^T   P^T goes from the accumulator registers straight into the second
+//            operand: the matrix core does not care how the 32 keys of a step are numbered
+//            as long as both operands agree, so Vt holds, for lane group kq, the keys
+//            kq*4 .. +3 and 16 + kq*4 .. +3 side by side at columns kq*8 .. +7
+// Ranges of keys (`nsplit` > 1) leave (maximum on the natural scale, sum, accumulator) for
+// latent_combine; the sink joins the denominator once, here or there.
+// WS, RT: the most 32-element steps of a row and 16-element tiles of the latent that the
+// instance holds in registers.
+#define LM_KT 32
+#define LM_VS (LM_KT + 8)
+#define LM_LOG2E 1.4426950408889634f
+#define LM_LN2 0.6931471805599453f
+
+template <int WS, int RT, int NW>
+__global__ void __launch_bounds__(NW * 64)
+latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                             const bf16_t* __restrict__ plane, long long page_stride,
+                             const int* __restrict__ block_table, int bt_stride,
+                             const int* __restrict__ positions, const int* __restrict__ wi_seq,
+                             const int* __restrict__ wi_row0, const int* __restrict__ wi_count,
+                             float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
+                             int HC, int W, int R, int page_size, float scale_log2,
+                             int keys_per_split, int nsplit, const float* __restrict__ sink) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lm_lds[];
+  constexpr int NT = NW * 64;
+  const int ws = (W + 31) / 32, rt = (R + 15) / 16;
+  const int KS = ws * 32 + 8;                       // elements from row to row of Ks
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lm_lds);   // [LM_KT][KS]
+  bf16_t* Vt = Ks + LM_KT * KS;                     // [rt * 16][LM_VS]
+
+  const int item = blockIdx.x, z = blockIdx.z;
+  const int h0 = blockIdx.y * HC;
+  const int G = min(HC, H - h0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int seq = wi_seq[item];
+  const int row0 = wi_row0[item];
+  int count = wi_count[item];
+  if (count * G > NW * 16) count = NW * 16 / G;     // the host never asks for more
+  const int rows = count * G;
+  const int* table = block_table + (size_t)seq * bt_stride;
+  const int hi = positions[row0 + count - 1];       // inclusive
+  int range_lo = z * keys_per_split;
+  int range_hi = range_lo + keys_per_split - 1;
+  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
+  if (range_hi > hi) range_hi = hi;
+
+  // columns of Ks beyond W and rows of Vt beyond R stay zero: clear everything once
+  {
+    const int words = (LM_KT * KS + rt * 16 * LM_VS) / 2;
+    uint32_t* w = reinterpret_cast<uint32_t*>(lm_lds);
+    for (int i = tid; i < words; i += NT) w[i] = 0u;
+  }
+
+  const int my = wave * 16 + r16;
+  const bool row_ok = my < rows;
+  const bool wave_on = wave * 16 < rows;
+  const int tok = row0 + (row_ok ? my / G : 0);
+  const int h = h0 + (row_ok ? my % G : 0);
+  const int pos_q = row_ok ? positions[tok] : -1;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8_t qf[WS];
+#pragma unroll
+  for (int ks = 0; ks < WS; ++ks) {
+    const int c = ks * 32 + kq * 8;
+    qf[ks] = (row_ok && c < W)
+                 ? *reinterpret_cast<const bf16x8_t*>(q + ((size_t)tok * H + h) * W + c)
+                 : zero8;
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int nchunk = R / 8, rchunk = (W - R) / 8;
+  for (int tile0 = range_lo; tile0 <= range_hi; tile0 += LM_KT) {
+    __syncthreads();      // the tile before is used up (first time: the clearing is done)
+    for (int blk = tid; blk < 4 * nchunk; blk += NT) {
+      const int c = blk % nchunk, g = blk / nchunk;
+      bf16x8_t a[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4);
+        const int kp = tile0 + key;
+        a[j] = zero8;
+        if (kp <= range_hi) {
+          const int page = table[kp / page_size];
+          if (page >= 0)
+            a[j] = *reinterpret_cast<const bf16x8_t*>(
+                plane + (size_t)page * page_stride + (size_t)(kp % page_size) * W + c * 8);
+        }
+        *reinterpret_cast<bf16x8_t*>(Ks + key * KS + c * 8) = a[j];
+      }
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        bf16x8_t t;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = a[j][r];
+        *reinterpret_cast<bf16x8_t*>(Vt + (c * 8 + r) * LM_VS + g * 8) = t;
+      }
+    }
+    for (int i = tid; i < LM_KT * rchunk; i += NT) {
+      const int key = i / rchunk, c = i % rchunk;
+      const int kp = tile0 + key;
+      bf16x8_t v = zero8;
+      if (kp <= range_hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          v = *reinterpret_cast<const bf16x8_t*>(
+              plane + (size_t)page * page_stride + (size_t)(kp % page_size) * W + R + c * 8);
+      }
+      *reinterpret_cast<bf16x8_t*>(Ks + key * KS + R + c * 8) = v;
+    }
+    __syncthreads();
+    if (!wave_on) continue;
+
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < WS; ++ks) {
+      if (ks < ws) {
+        const bf16x8_t k0 = *reinterpret_cast<const bf16x8_t*>(Ks + r16 * KS + ks * 32 + kq * 8);
+        const bf16x8_t k1 =
+            *reinterpret_cast<const bf16x8_t*>(Ks + (16 + r16) * KS + ks * 32 + kq * 8);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[ks], s1, 0, 0, 0);
+      }
+    }
+    float sc[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int kp = tile0 + (i < 4 ? kq * 4 + i : 16 + kq * 4 + (i - 4));
+      const float v = (i < 4 ? s0[i] : s1[i - 4]) * scale_log2;
+      sc[i] = (kp <= pos_q && kp <= range_hi) ? v : -INFINITY;
+      tmax = fmaxf(tmax, sc[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = m_new > -INFINITY ? m_new : 0.f;
+    const float alpha = exp2f(m - m_use);
+    bf16x8_t pf;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bf16_t pb = (bf16_t)exp2f(sc[i] - m_use);
+      pf[i] = pb;
+      psum += (float)pb;
+    }
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      if (t < rt) {
+        const bf16x8_t vf =
+            *reinterpret_cast<const bf16x8_t*>(Vt + (t * 16 + r16) * LM_VS + kq * 8);
+        f32x4_t acc = o[t];
+        acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc, 0, 0, 0);
+      }
+    }
+  }
+
+  if (!wave_on) return;
+  float lt = l;
+  lt += __shfl_xor(lt, 16, 64);
+  lt += __shfl_xor(lt, 32, 64);
+  if (!row_ok) return;
+  if (nsplit == 1) {
+    if (sink) lt += exp2f(sink[h] * LM_LOG2E - m);
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    bf16_t* orow = out + ((size_t)tok * H + h) * R;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const int r = t * 16 + kq * 4;
+      if (t < rt && r < R) {
+        bf16x4_t v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[t][i] * inv);
+        *reinterpret_cast<bf16x4_t*>(orow + r) = v;
+      }
+    }
+  } else {
+    const size_t pidx = ((size_t)tok * H + h) * nsplit + z;
+    float* pa = part_acc + pidx * R;
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      const int r = t * 16 + kq * 4;
+      if (t < rt && r < R) *reinterpret_cast<f32x4_t*>(pa + r) = o[t];
+    }
+    if (kq == 0) {
+      part_ml[pidx * 2] = m * LM_LN2;
+      part_ml[pidx * 2 + 1] = lt;
+    }
+  }
+}
+
 // The partial results of a row's ranges -> the row.  `base2`: the partial maxima are whole
 // numbers on the base-2 scale (what the matrix-core kernel keeps), so a partial result's
 // weight 2^(m_z - m) is an exact power of two.
@@ -562,6 +773,75 @@ static int launch_latent_attention(const void* q, void* out, const void* plane,
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)plane,
                      page_stride, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
                      part_acc, part_ml, H, HC, W, R, page_size, scale, keys_per_split, nsplit, sink);
+  return za_launch_status();
+}
+
+template <int WS, int RT, int NW>
+static int launch_latent_mfma(const void* q, void* out, const void* plane, long long page_stride,
+                              const int* block_table, int bt_stride, const int* positions,
+                              const int* wi_seq, const int* wi_row0, const int* wi_count,
+                              int n_items, float* part_acc, float* part_ml, int H, int W, int R,
+                              int page_size, float scale, int keys_per_split, int nsplit,
+                              const float* sink, hipStream_t stream) {
+  const int ws = (W + 31) / 32, rt = (R + 15) / 16;
+  const size_t shmem = ((size_t)LM_KT * (ws * 32 + 8) + (size_t)rt * 16 * LM_VS) * sizeof(bf16_t);
+  auto kernel = latent_attention_mfma_kernel<WS, RT, NW>;
+  static size_t allowed = 0;
+  if (shmem > allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (e != hipSuccess) return (int)e;
+    allowed = shmem;
+  }
+  const int HC = H < NW * 16 ? H : NW * 16;
+  dim3 grid(n_items, (H + HC - 1) / HC, nsplit), block(NW * 64);
+  hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const bf16_t*)q, (bf16_t*)out,
+                     (const bf16_t*)plane, page_stride, block_table, bt_stride, positions, wi_seq,
+                     wi_row0, wi_count, part_acc, part_ml, H, HC, W, R, page_size,
+                     scale * LM_LOG2E, keys_per_split, nsplit, sink);
+  return za_launch_status();
+}
+
+// The matrix-core form: bfloat16, `width` and `kv_rank` multiples of 8.  `waves`: 4 (work
+// items of at most 64 / min(heads, 64) tokens) or 1 (single tokens, as a step that only
+// decodes has; heads in chunks of 16).  Arguments otherwise as za_latent_attention.
+extern "C" int za_latent_attention_mfma(const void* q, void* out, const void* plane,
+                                        long long page_stride, const int* block_table,
+                                        int bt_stride, const int* positions, const int* wi_seq,
+                                        const int* wi_row0, const int* wi_count, int n_items,
+                                        int n_tokens, float* part_acc, float* part_ml, int heads,
+                                        int width, int kv_rank, int page_size, float scale,
+                                        int keys_per_split, int nsplit, const float* sink,
+                                        int waves, hipStream_t stream) {
+  if (n_items == 0 || n_tokens == 0) return 0;
+  if (n_items < 0 || heads <= 0 || width <= 0 || kv_rank <= 0 || kv_rank > width ||
+      page_size <= 0 || bt_stride <= 0 || nsplit < 1 || !q || !out || !plane || !block_table ||
+      !positions || !wi_seq || !wi_row0 || !wi_count ||
+      page_stride < (long long)page_size * width || (waves != 1 && waves != 4))
+    return ZA_ERR_ARG;
+  if (width % 8 || kv_rank % 8 || width > LA_MAX_W || kv_rank > LA_MAX_R || nsplit > 65535)
+    return ZA_ERR_UNSUPPORTED;
+  if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
+    return ZA_ERR_ARG;
+  const int ws = (width + 31) / 32, rt = (kv_rank + 15) / 16;
+  int rc;
+#define ZA_LM_ARGS                                                                              \
+  q, out, plane, page_stride, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,     \
+      n_items, part_acc, part_ml, heads, width, kv_rank, page_size, scale, keys_per_split,      \
+      nsplit, sink, stream
+  if (ws <= 6 && rt <= 8)
+    rc = waves == 4 ? launch_latent_mfma<6, 8, 4>(ZA_LM_ARGS) : launch_latent_mfma<6, 8, 1>(ZA_LM_ARGS);
+  else if (ws <= 10 && rt <= 16)
+    rc = waves == 4 ? launch_latent_mfma<10, 16, 4>(ZA_LM_ARGS)
+                    : launch_latent_mfma<10, 16, 1>(ZA_LM_ARGS);
+  else
+    rc = waves == 4 ? launch_latent_mfma<18, 32, 4>(ZA_LM_ARGS)
+                    : launch_latent_mfma<18, 32, 1>(ZA_LM_ARGS);
+#undef ZA_LM_ARGS
+  if (rc != 0 || nsplit == 1) return rc;
+  dim3 grid((unsigned)((size_t)n_tokens * heads)), block(64);
+  hipLaunchKernelGGL((latent_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc, part_ml,
+                     (bf16_t*)out, kv_rank, nsplit, 0, sink, heads);
   return za_launch_status();
 }
 

@@ -170,6 +170,10 @@ _SIGNATURES = {
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                         c_float, c_int, c_int, c_void_p, c_void_p],
+    ("latent", "za_latent_attention_mfma"): [c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
+                                             c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                             c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                             c_float, c_int, c_int, c_void_p, c_int, c_void_p],
 }
 _functions = {}
 
@@ -2181,6 +2185,7 @@ def normed_add_(stream: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps
 
 # ------------------------------------------------------------ latent attention
 LATENT_MAX_ROWS = 32        # rows (token, head) of a work item of the general kernel
+LATENT_MFMA_ROWS = 64       # of the matrix-core kernel with four waves (16 with one)
 LATENT_MAX_WIDTH = 576      # cached elements a token
 LATENT_MAX_RANK = 512       # of which the latent
 
@@ -2312,11 +2317,14 @@ def latent_attention(q: torch.Tensor, plane: torch.Tensor, kv_rank: int, block_t
                      positions: torch.Tensor, item_seq: torch.Tensor, item_row0: torch.Tensor,
                      item_count: torch.Tensor, n_items: int, scale: float,
                      sink: Optional[torch.Tensor] = None, keys_per_split: int = 0,
-                     nsplit: int = 1) -> torch.Tensor:
+                     nsplit: int = 1, waves: int = 0) -> torch.Tensor:
     """Causal attention of the folded queries ``q [T, heads, width]`` over cached rows of
     ``width`` elements whose first ``kv_rank`` are also the values; returns ``[T, heads,
     kv_rank]``.  ``item_*``: work items of at most ``LATENT_MAX_ROWS // min(heads,
-    LATENT_MAX_ROWS)`` consecutive rows of one request.  ``sink``: 32-bit ``[heads]``."""
+    LATENT_MAX_ROWS)`` consecutive rows of one request.  ``sink``: 32-bit ``[heads]``.
+    ``waves``: 0 is the general kernel; 4 or 1 the matrix-core kernel (``latent_mfma_fits``)
+    with work items of at most ``LATENT_MFMA_ROWS // min(heads, LATENT_MFMA_ROWS)`` tokens
+    (4 waves) or of single tokens (1 wave)."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, width], got {tuple(q.shape)}")
     T, H, W = q.shape
@@ -2342,11 +2350,29 @@ def latent_attention(q: torch.Tensor, plane: torch.Tensor, kv_rank: int, block_t
             raise KernelError("keys_per_split must be a positive multiple of 64")
         part_acc = torch.empty((T, H, nsplit, kv_rank), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, H, nsplit, 2), dtype=torch.float32, device=q.device)
-    rc = _fn("latent", "za_latent_attention")(
-        _ptr(q), _ptr(out), _ptr(plane), stride, _ptr(block_table), block_table.shape[1],
-        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
-        _ptr(part_acc), _ptr(part_ml), _code(q.dtype), H, W, int(kv_rank), page_size, float(scale),
-        int(keys_per_split), int(nsplit), _ptr(sink), _stream())
+    if waves:
+        if waves not in (1, 4) or not latent_mfma_fits(q.dtype, W, kv_rank) or stride % 8 \
+                or plane.data_ptr() % 16 or q.data_ptr() % 16:
+            raise KernelError(f"the matrix-core latent attention takes bfloat16 rows of multiples "
+                              f"of 8 elements and 1 or 4 waves, got {q.dtype}, {W}, {kv_rank}, {waves}")
+        rc = _fn("latent", "za_latent_attention_mfma")(
+            _ptr(q), _ptr(out), _ptr(plane), stride, _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), H, W, int(kv_rank), page_size, float(scale),
+            int(keys_per_split), int(nsplit), _ptr(sink), int(waves), _stream())
+    else:
+        rc = _fn("latent", "za_latent_attention")(
+            _ptr(q), _ptr(out), _ptr(plane), stride, _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), _code(q.dtype), H, W, int(kv_rank), page_size,
+            float(scale), int(keys_per_split), int(nsplit), _ptr(sink), _stream())
     _check(rc, "latent_attention")
-    _note("attention", kernel="latent", rows=T, dtype=q.dtype, nsplit=int(nsplit))
+    _note("attention", kernel="latent_mfma" if waves else "latent", rows=T, dtype=q.dtype,
+          nsplit=int(nsplit), waves=int(waves))
     return out
+
+
+def latent_mfma_fits(dtype, width: int, kv_rank: int) -> bool:
+    """Whether the matrix-core latent attention takes these rows: bfloat16, 16-byte pieces."""
+    return dtype == torch.bfloat16 and width % 8 == 0 and kv_rank % 8 == 0 \
+        and width <= LATENT_MAX_WIDTH and kv_rank <= LATENT_MAX_RANK

@@ -37,6 +37,26 @@ from .base import Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer
 from .feed_forward import fuse_rows, pad_rows
 
 
+LATENT_SPLIT_TARGET = 1024    # workgroups to reach by cutting contexts into ranges
+LATENT_SPLIT_KEYS = 128       # keys of a range at least
+LATENT_SPLIT_BYTES = 32 << 20  # the most that the ranges' partial results may take
+
+
+def plan_latent_split(groups: int, max_keys: int):
+    """(keys per range, number of ranges) for one launch of the matrix-core kernel: a function
+    of the batch shape and of the longest context only.  A workgroup holds one or four waves
+    and takes 32 keys a tile, so short ranges pay: as many as reach ``LATENT_SPLIT_TARGET``
+    workgroups, of at least ``LATENT_SPLIT_KEYS`` keys each."""
+    if groups >= LATENT_SPLIT_TARGET or max_keys <= 2 * LATENT_SPLIT_KEYS:
+        return 0, 1
+    nsplit = min(LATENT_SPLIT_TARGET // groups, max_keys // LATENT_SPLIT_KEYS, 64)
+    if nsplit <= 1:
+        return 0, 1
+    keys = ((max_keys + nsplit - 1) // nsplit + 63) // 64 * 64
+    nsplit = (max_keys + keys - 1) // keys
+    return (keys, nsplit) if nsplit > 1 else (0, 1)
+
+
 class LatentAttention(Mixer):
     kind = "latent_attention"
     graph_safe = True
@@ -123,7 +143,10 @@ class LatentAttention(Mixer):
         if v_up.dtype == torch.bfloat16 and R % 8:
             v_up = v_up.float()
         self.k_fold, self.v_expand = k_up, v_up
-        self.rows_per_item = max(1, ops.LATENT_MAX_ROWS // min(nh, ops.LATENT_MAX_ROWS))
+        # bfloat16 rows of 16-byte pieces run on the matrix cores, in work items of 64 rows
+        self.mfma = ops.latent_mfma_fits(runtime.dtype, self.width, R)
+        most = ops.LATENT_MFMA_ROWS if self.mfma else ops.LATENT_MAX_ROWS
+        self.rows_per_item = max(1, most // min(nh, most))
         self.item_granularities = [self.rows_per_item]
         for w, what in ((self.w_open, "w_open"), (self.w_q_up, "w_q_up"), (self.w_out, "w_out")):
             ops.check_projection_weight(w, "latent attention " + what)
@@ -146,10 +169,20 @@ class LatentAttention(Mixer):
             ops.rotate_part_(q, d, qf, R, dr, step.positions, self.inv_freq, self.rot_dims,
                              self.adjacent)
         item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
-        keys, nsplit = plan_split(n_items, 1, step.max_keys)
+        waves = 0
+        if self.mfma:
+            # a step that only decodes: a wave a workgroup, heads in chunks of 16
+            waves = 1 if step.n_tokens == step.n_seqs else 4
+            keys, nsplit = plan_latent_split(n_items * (-(-nh // (16 * waves))), step.max_keys)
+            # (the ranges' partial results are 32-bit rows of the latent's width: no cut where
+            # they would be larger than the step is worth)
+            if T * nh * nsplit * R * 4 > LATENT_SPLIT_BYTES:
+                keys, nsplit = 0, 1
+        else:
+            keys, nsplit = plan_split(n_items, 1, step.max_keys)
         o = ops.latent_attention(qf, plane, R, step.block_tables[cache.group], step.positions,
                                  item_seq, item_row0, item_count, n_items, self.scale, self.sink,
-                                 keys, nsplit)
+                                 keys, nsplit, waves)
         # every head's result expanded by its Wuv, times the gate
         a = ops.head_linear(o, 0, self.v_expand, gate=down if self.gate else None,
                             gate_col=self.gate_col, gate_mode=self.gate)
