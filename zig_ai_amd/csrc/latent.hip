@@ -502,15 +502,15 @@ latent_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* _
 
 // ------------------------------------------------------------ latent_attention_mfma
 // bfloat16 on the matrix cores, rows of W and latents of R elements that are multiples of 8
-// (16-byte pieces).  A workgroup of NW waves serves one work item and one chunk of heads,
-// at most NW * 16 rows (token, head); each wave owns 16 of them.  Per tile of 32 keys:
+// (16-byte pieces).  Per tile of 32 keys:
 //   staging  every thread fetches, for 8 keys, the same 8 latent elements (eight 16-byte
 //            loads), stores them as they are into Ks [32][W] and, turned round in its
 //            registers, into Vt [R][32]: the second product wants, for one latent element,
-//            consecutive keys side by side.  The rotated key part goes into Ks only.
-//   S^T = K Q^T   keys are the rows of the first operand, the wave's 16 query rows the
-//            columns: a lane ends up with ONE query row's scores for keys kq*4 .. +3 of
-//            each half of the tile (kq = lane / 16)
+//            consecutive keys side by side.  The rotated key part goes into Ks only.  The
+//            loads of the next tile are issued before the products of this one.
+//   S^T = K Q^T   keys are the rows of the first operand, 16 query rows the columns: a lane
+//            ends up with ONE query row's scores for keys kq*4 .. +3 of each half of the
+//            tile (kq = lane / 16)
 //   p = 2^(s * scale * log2(e) - m) in 32-bit, the running maximum shared by the four lanes
 //            of a query row; p is rounded to bfloat16 and the sum that normalises the result
 //            is the sum of the rounded values
@@ -518,31 +518,164 @@ latent_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* _
 //            operand: the matrix core does not care how the 32 keys of a step are numbered
 //            as long as both operands agree, so Vt holds, for lane group kq, the keys
 //            kq*4 .. +3 and 16 + kq*4 .. +3 side by side at columns kq*8 .. +7
+// Two kernels share this.  latent_attention_mfma_kernel: a workgroup of four waves serves
+// one work item and one chunk of heads, at most 64 rows (token, head), 16 a wave.
+// latent_decode_mfma_kernel: work items of at most 16 rows (single tokens times a chunk of
+// 16 heads) that all four waves share: a wave takes every fourth 32-element step of the
+// first product (the partial scores are added up through LDS, in a fixed order, so every
+// wave holds the same scores) and every fourth 16-element tile of the result.
 // Ranges of keys (`nsplit` > 1) leave (maximum on the natural scale, sum, accumulator) for
 // latent_combine; the sink joins the denominator once, here or there.
-// WS, RT: the most 32-element steps of a row and 16-element tiles of the latent that the
+// WS, RT: the most 32-element steps of a row and 16-element tiles of the latent that an
 // instance holds in registers.
 #define LM_KT 32
 #define LM_VS (LM_KT + 8)
+#define LM_NT 256
+// Vt holds latent element e at row (e % 8) * P + e / 8, P = lm_vp(tiles of 16 elements): the
+// threads of a wave store eight neighbouring rows each, at neighbouring e / 8, and a fragment
+// reads 16 neighbouring e; with P = 2 (mod 16) and rows of 80 bytes neither meets a bank twice.
+__host__ __device__ __forceinline__ int lm_vp(int rt) { return (2 * rt - 2 + 15) / 16 * 16 + 2; }
 #define LM_LOG2E 1.4426950408889634f
 #define LM_LN2 0.6931471805599453f
 
-template <int WS, int RT, int NW>
-__global__ void __launch_bounds__(NW * 64)
+struct LmTile {
+  bf16x8_t a[8];   // 8 keys x the same 8 latent elements
+  bf16x8_t rot;    // 8 elements of one key's rotated part
+};
+
+struct LmCache {
+  const bf16_t* plane;
+  long long page_stride;
+  const int* table;
+  int page_size, shift;   // shift: log2(page_size), or -1
+  int W, R;
+};
+
+// The page of key position `kp` (clamped into the range, so the entry exists) and the key's
+// place in it: loads that depend on nothing but the tile, issued for all keys at once.
+__device__ __forceinline__ int lm_page(const LmCache& c, int kp, int& off) {
+  if (c.shift >= 0) {
+    off = kp & (c.page_size - 1);
+    return c.table[kp >> c.shift];
+  }
+  off = kp % c.page_size;
+  return c.table[kp / c.page_size];
+}
+
+// Key `j` of the eight that lane group `g` feeds the second product side by side.
+__device__ __forceinline__ int lm_key(int g, int j) { return j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4); }
+
+// No branch between the loads: a key beyond the range reads the range's last key, a page
+// that is not there reads page 0, and the value is dropped afterwards.
+__device__ __forceinline__ void lm_fetch(LmTile& t, const LmCache& c, int tile0, int range_hi, int tid) {
+  const int nchunk = c.R / 8, rchunk = (c.W - c.R) / 8;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (tid < 4 * nchunk) {          // R <= 512: a block a thread at most
+    const int ch = tid % nchunk, g = tid / nchunk;
+    int page[8], off[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) page[j] = lm_page(c, min(tile0 + lm_key(g, j), range_hi), off[j]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      t.a[j] = *reinterpret_cast<const bf16x8_t*>(
+          c.plane + (size_t)max(page[j], 0) * c.page_stride + (size_t)off[j] * c.W + ch * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (tile0 + lm_key(g, j) > range_hi || page[j] < 0) t.a[j] = zero8;
+  }
+  t.rot = zero8;
+  if (tid < LM_KT * rchunk) {
+    const int kp = tile0 + tid / rchunk;
+    int off;
+    const int page = lm_page(c, min(kp, range_hi), off);
+    const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(
+        c.plane + (size_t)max(page, 0) * c.page_stride + (size_t)off * c.W + c.R + (tid % rchunk) * 8);
+    if (kp <= range_hi && page >= 0) t.rot = v;
+  }
+}
+
+__device__ __forceinline__ void lm_store(const LmTile& t, const LmCache& c, bf16_t* Ks, bf16_t* Vt,
+                                         int KS, int VP, int tile0, int range_hi, int tid) {
+  const int nchunk = c.R / 8, rchunk = (c.W - c.R) / 8;
+  if (tid < 4 * nchunk) {
+    const int ch = tid % nchunk, g = tid / nchunk;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *reinterpret_cast<bf16x8_t*>(Ks + lm_key(g, j) * KS + ch * 8) = t.a[j];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      bf16x8_t v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = t.a[j][r];
+      *reinterpret_cast<bf16x8_t*>(Vt + (r * VP + ch) * LM_VS + g * 8) = v;
+    }
+  }
+  if (tid < LM_KT * rchunk)
+    *reinterpret_cast<bf16x8_t*>(Ks + (tid / rchunk) * KS + c.R + (tid % rchunk) * 8) = t.rot;
+  // a rotated part of more than 64 elements: the rest, not fetched ahead
+  for (int i = tid + LM_NT; i < LM_KT * rchunk; i += LM_NT) {
+    const int key = i / rchunk, kp = tile0 + key;
+    bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (kp <= range_hi) {
+      int off;
+      const int page = lm_page(c, kp, off);
+      if (page >= 0)
+        v = *reinterpret_cast<const bf16x8_t*>(c.plane + (size_t)page * c.page_stride +
+                                               (size_t)off * c.W + c.R + (i % rchunk) * 8);
+    }
+    *reinterpret_cast<bf16x8_t*>(Ks + key * KS + c.R + (i % rchunk) * 8) = v;
+  }
+}
+
+// One query row's scores of a tile (this lane's eight keys) -> its probabilities as the
+// second operand's fragment; updates the running maximum and sum; returns the factor the
+// accumulator takes.
+__device__ __forceinline__ float lm_softmax(const f32x4_t& s0, const f32x4_t& s1, int tile0, int kq,
+                                            int pos_q, int range_hi, float scale_log2, float& m,
+                                            float& l, bf16x8_t& pf) {
+  float sc[8];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int kp = tile0 + lm_key(kq, i);
+    const float v = (i < 4 ? s0[i] : s1[i - 4]) * scale_log2;
+    sc[i] = (kp <= pos_q && kp <= range_hi) ? v : -INFINITY;
+    tmax = fmaxf(tmax, sc[i]);
+  }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+  const float m_new = fmaxf(m, tmax);
+  const float m_use = m_new > -INFINITY ? m_new : 0.f;
+  const float alpha = m == m_new ? 1.0f : exp2f(m - m_use);
+  float psum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const bf16_t pb = (bf16_t)exp2f(sc[i] - m_use);
+    pf[i] = pb;
+    psum += (float)pb;
+  }
+  l = l * alpha + psum;
+  m = m_new;
+  return alpha;
+}
+
+template <int WS, int RT>
+__global__ void __launch_bounds__(LM_NT)
 latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                              const bf16_t* __restrict__ plane, long long page_stride,
                              const int* __restrict__ block_table, int bt_stride,
                              const int* __restrict__ positions, const int* __restrict__ wi_seq,
                              const int* __restrict__ wi_row0, const int* __restrict__ wi_count,
                              float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
-                             int HC, int W, int R, int page_size, float scale_log2,
-                             int keys_per_split, int nsplit, const float* __restrict__ sink) {
+                             int HC, int W, int R, int page_size, int page_shift,
+                             float scale_log2, int keys_per_split, int nsplit,
+                             const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lm_lds[];
-  constexpr int NT = NW * 64;
   const int ws = (W + 31) / 32, rt = (R + 15) / 16;
   const int KS = ws * 32 + 8;                       // elements from row to row of Ks
   bf16_t* Ks = reinterpret_cast<bf16_t*>(lm_lds);   // [LM_KT][KS]
-  bf16_t* Vt = Ks + LM_KT * KS;                     // [rt * 16][LM_VS]
+  bf16_t* Vt = Ks + LM_KT * KS;                     // [8 * VP][LM_VS]
+  const int VP = lm_vp(rt);
 
   const int item = blockIdx.x, z = blockIdx.z;
   const int h0 = blockIdx.y * HC;
@@ -552,20 +685,21 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
   const int seq = wi_seq[item];
   const int row0 = wi_row0[item];
   int count = wi_count[item];
-  if (count * G > NW * 16) count = NW * 16 / G;     // the host never asks for more
+  if (count * G > 64) count = 64 / G;               // the host never asks for more
   const int rows = count * G;
-  const int* table = block_table + (size_t)seq * bt_stride;
   const int hi = positions[row0 + count - 1];       // inclusive
   int range_lo = z * keys_per_split;
   int range_hi = range_lo + keys_per_split - 1;
   if (nsplit == 1) { range_lo = 0; range_hi = hi; }
   if (range_hi > hi) range_hi = hi;
+  const LmCache cache = {plane, page_stride, block_table + (size_t)seq * bt_stride, page_size,
+                         page_shift, W, R};
 
   // columns of Ks beyond W and rows of Vt beyond R stay zero: clear everything once
   {
-    const int words = (LM_KT * KS + rt * 16 * LM_VS) / 2;
+    const int words = (LM_KT * KS + 8 * VP * LM_VS) / 2;
     uint32_t* w = reinterpret_cast<uint32_t*>(lm_lds);
-    for (int i = tid; i < words; i += NT) w[i] = 0u;
+    for (int i = tid; i < words; i += LM_NT) w[i] = 0u;
   }
 
   const int my = wave * 16 + r16;
@@ -588,91 +722,41 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
 #pragma unroll
   for (int t = 0; t < RT; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int nchunk = R / 8, rchunk = (W - R) / 8;
+  LmTile regs;
+  if (range_lo <= range_hi) lm_fetch(regs, cache, range_lo, range_hi, tid);
   for (int tile0 = range_lo; tile0 <= range_hi; tile0 += LM_KT) {
     __syncthreads();      // the tile before is used up (first time: the clearing is done)
-    for (int blk = tid; blk < 4 * nchunk; blk += NT) {
-      const int c = blk % nchunk, g = blk / nchunk;
-      bf16x8_t a[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4);
-        const int kp = tile0 + key;
-        a[j] = zero8;
-        if (kp <= range_hi) {
-          const int page = table[kp / page_size];
-          if (page >= 0)
-            a[j] = *reinterpret_cast<const bf16x8_t*>(
-                plane + (size_t)page * page_stride + (size_t)(kp % page_size) * W + c * 8);
-        }
-        *reinterpret_cast<bf16x8_t*>(Ks + key * KS + c * 8) = a[j];
-      }
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        bf16x8_t t;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) t[j] = a[j][r];
-        *reinterpret_cast<bf16x8_t*>(Vt + (c * 8 + r) * LM_VS + g * 8) = t;
-      }
-    }
-    for (int i = tid; i < LM_KT * rchunk; i += NT) {
-      const int key = i / rchunk, c = i % rchunk;
-      const int kp = tile0 + key;
-      bf16x8_t v = zero8;
-      if (kp <= range_hi) {
-        const int page = table[kp / page_size];
-        if (page >= 0)
-          v = *reinterpret_cast<const bf16x8_t*>(
-              plane + (size_t)page * page_stride + (size_t)(kp % page_size) * W + R + c * 8);
-      }
-      *reinterpret_cast<bf16x8_t*>(Ks + key * KS + R + c * 8) = v;
-    }
+    lm_store(regs, cache, Ks, Vt, KS, VP, tile0, range_hi, tid);
     __syncthreads();
-    if (!wave_on) continue;
-
-    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    if (tile0 + LM_KT <= range_hi) lm_fetch(regs, cache, tile0 + LM_KT, range_hi, tid);
+    if (wave_on) {
+      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < WS; ++ks) {
-      if (ks < ws) {
-        const bf16x8_t k0 = *reinterpret_cast<const bf16x8_t*>(Ks + r16 * KS + ks * 32 + kq * 8);
-        const bf16x8_t k1 =
-            *reinterpret_cast<const bf16x8_t*>(Ks + (16 + r16) * KS + ks * 32 + kq * 8);
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[ks], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[ks], s1, 0, 0, 0);
+      for (int ks = 0; ks < WS; ++ks) {
+        if (ks < ws) {
+          const bf16x8_t k0 =
+              *reinterpret_cast<const bf16x8_t*>(Ks + r16 * KS + ks * 32 + kq * 8);
+          const bf16x8_t k1 =
+              *reinterpret_cast<const bf16x8_t*>(Ks + (16 + r16) * KS + ks * 32 + kq * 8);
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[ks], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[ks], s1, 0, 0, 0);
+        }
       }
-    }
-    float sc[8];
-    float tmax = -INFINITY;
+      bf16x8_t pf;
+      const float alpha = lm_softmax(s0, s1, tile0, kq, pos_q, range_hi, scale_log2, m, l, pf);
+      if (!__all(alpha == 1.0f)) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int kp = tile0 + (i < 4 ? kq * 4 + i : 16 + kq * 4 + (i - 4));
-      const float v = (i < 4 ? s0[i] : s1[i - 4]) * scale_log2;
-      sc[i] = (kp <= pos_q && kp <= range_hi) ? v : -INFINITY;
-      tmax = fmaxf(tmax, sc[i]);
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
-    const float m_use = m_new > -INFINITY ? m_new : 0.f;
-    const float alpha = exp2f(m - m_use);
-    bf16x8_t pf;
-    float psum = 0.f;
+        for (int t = 0; t < RT; ++t) {
+          if (t < rt) { o[t][0] *= alpha; o[t][1] *= alpha; o[t][2] *= alpha; o[t][3] *= alpha; }
+        }
+      }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const bf16_t pb = (bf16_t)exp2f(sc[i] - m_use);
-      pf[i] = pb;
-      psum += (float)pb;
-    }
-    l = l * alpha + psum;
-    m = m_new;
-#pragma unroll
-    for (int t = 0; t < RT; ++t) {
-      if (t < rt) {
-        const bf16x8_t vf =
-            *reinterpret_cast<const bf16x8_t*>(Vt + (t * 16 + r16) * LM_VS + kq * 8);
-        f32x4_t acc = o[t];
-        acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc, 0, 0, 0);
+      for (int t = 0; t < RT; ++t) {
+        if (t < rt) {
+          const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
+              Vt + ((r16 & 7) * VP + 2 * t + (r16 >> 3)) * LM_VS + kq * 8);
+          o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[t], 0, 0, 0);
+        }
       }
     }
   }
@@ -705,6 +789,153 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
       if (t < rt && r < R) *reinterpret_cast<f32x4_t*>(pa + r) = o[t];
     }
     if (kq == 0) {
+      part_ml[pidx * 2] = m * LM_LN2;
+      part_ml[pidx * 2 + 1] = lt;
+    }
+  }
+}
+
+template <int WS, int RT>
+__global__ void __launch_bounds__(LM_NT)
+latent_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                          const bf16_t* __restrict__ plane, long long page_stride,
+                          const int* __restrict__ block_table, int bt_stride,
+                          const int* __restrict__ positions, const int* __restrict__ wi_seq,
+                          const int* __restrict__ wi_row0, const int* __restrict__ wi_count,
+                          float* __restrict__ part_acc, float* __restrict__ part_ml, int H, int HC,
+                          int W, int R, int page_size, int page_shift, float scale_log2,
+                          int keys_per_split, int nsplit, const float* __restrict__ sink) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lm_lds[];
+  constexpr int QW = (WS + 3) / 4, OT = (RT + 3) / 4;
+  const int ws = (W + 31) / 32, rt = (R + 15) / 16;
+  const int KS = ws * 32 + 8;
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lm_lds);   // [LM_KT][KS]
+  bf16_t* Vt = Ks + LM_KT * KS;                     // [8 * VP][LM_VS]
+  const int VP = lm_vp(rt);
+  float* Sx = reinterpret_cast<float*>(Vt + 8 * lm_vp(rt) * LM_VS);   // [4 waves][64 lanes][8]
+
+  const int item = blockIdx.x, z = blockIdx.z;
+  const int h0 = blockIdx.y * HC;
+  const int G = min(HC, H - h0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int seq = wi_seq[item];
+  const int row0 = wi_row0[item];
+  int count = wi_count[item];
+  if (count * G > 16) count = 16 / G;               // the host never asks for more
+  const int rows = count * G;
+  const int hi = positions[row0 + count - 1];       // inclusive
+  int range_lo = z * keys_per_split;
+  int range_hi = range_lo + keys_per_split - 1;
+  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
+  if (range_hi > hi) range_hi = hi;
+  const LmCache cache = {plane, page_stride, block_table + (size_t)seq * bt_stride, page_size,
+                         page_shift, W, R};
+  {
+    const int words = (LM_KT * KS + 8 * VP * LM_VS) / 2;
+    uint32_t* w = reinterpret_cast<uint32_t*>(lm_lds);
+    for (int i = tid; i < words; i += LM_NT) w[i] = 0u;
+  }
+
+  const bool row_ok = r16 < rows;
+  const int tok = row0 + (row_ok ? r16 / G : 0);
+  const int h = h0 + (row_ok ? r16 % G : 0);
+  const int pos_q = row_ok ? positions[tok] : -1;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8_t qf[QW];          // the steps wave, wave + 4, ... of the row
+#pragma unroll
+  for (int j = 0; j < QW; ++j) {
+    const int c = (j * 4 + wave) * 32 + kq * 8;
+    qf[j] = (row_ok && c < W)
+                ? *reinterpret_cast<const bf16x8_t*>(q + ((size_t)tok * H + h) * W + c)
+                : zero8;
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[OT];            // the tiles wave, wave + 4, ... of the result
+#pragma unroll
+  for (int j = 0; j < OT; ++j) o[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  // two tiles are on their way while one is worked on: a step of few rows has little to do
+  // a tile, and what it waits for is memory
+  auto tile = [&](LmTile& regs, int tile0) {
+    __syncthreads();
+    lm_store(regs, cache, Ks, Vt, KS, VP, tile0, range_hi, tid);
+    __syncthreads();
+    if (tile0 + 2 * LM_KT <= range_hi) lm_fetch(regs, cache, tile0 + 2 * LM_KT, range_hi, tid);
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < QW; ++j) {
+      const int ks = j * 4 + wave;
+      if (ks < ws) {
+        const bf16x8_t k0 = *reinterpret_cast<const bf16x8_t*>(Ks + r16 * KS + ks * 32 + kq * 8);
+        const bf16x8_t k1 =
+            *reinterpret_cast<const bf16x8_t*>(Ks + (16 + r16) * KS + ks * 32 + kq * 8);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[j], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[j], s1, 0, 0, 0);
+      }
+    }
+    *reinterpret_cast<f32x4_t*>(Sx + (wave * 64 + lane) * 8) = s0;
+    *reinterpret_cast<f32x4_t*>(Sx + (wave * 64 + lane) * 8 + 4) = s1;
+    __syncthreads();
+    s0 = *reinterpret_cast<const f32x4_t*>(Sx + lane * 8);
+    s1 = *reinterpret_cast<const f32x4_t*>(Sx + lane * 8 + 4);
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(Sx + (w * 64 + lane) * 8);
+      const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(Sx + (w * 64 + lane) * 8 + 4);
+      s0[0] += a0[0]; s0[1] += a0[1]; s0[2] += a0[2]; s0[3] += a0[3];
+      s1[0] += a1[0]; s1[1] += a1[1]; s1[2] += a1[2]; s1[3] += a1[3];
+    }
+    bf16x8_t pf;
+    const float alpha = lm_softmax(s0, s1, tile0, kq, pos_q, range_hi, scale_log2, m, l, pf);
+#pragma unroll
+    for (int j = 0; j < OT; ++j) {
+      const int t = j * 4 + wave;
+      if (t < rt) {
+        const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
+            Vt + ((r16 & 7) * VP + 2 * t + (r16 >> 3)) * LM_VS + kq * 8);
+        f32x4_t acc = o[j];
+        acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+        o[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc, 0, 0, 0);
+      }
+    }
+  };
+  LmTile regs_a, regs_b;
+  if (range_lo <= range_hi) lm_fetch(regs_a, cache, range_lo, range_hi, tid);
+  if (range_lo + LM_KT <= range_hi) lm_fetch(regs_b, cache, range_lo + LM_KT, range_hi, tid);
+  for (int tile0 = range_lo; tile0 <= range_hi; tile0 += 2 * LM_KT) {
+    tile(regs_a, tile0);
+    if (tile0 + LM_KT > range_hi) break;
+    tile(regs_b, tile0 + LM_KT);
+  }
+
+  float lt = l;
+  lt += __shfl_xor(lt, 16, 64);
+  lt += __shfl_xor(lt, 32, 64);
+  if (!row_ok) return;
+  if (nsplit == 1) {
+    if (sink) lt += exp2f(sink[h] * LM_LOG2E - m);
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    bf16_t* orow = out + ((size_t)tok * H + h) * R;
+#pragma unroll
+    for (int j = 0; j < OT; ++j) {
+      const int t = j * 4 + wave, r = t * 16 + kq * 4;
+      if (t < rt && r < R) {
+        bf16x4_t v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[j][i] * inv);
+        *reinterpret_cast<bf16x4_t*>(orow + r) = v;
+      }
+    }
+  } else {
+    const size_t pidx = ((size_t)tok * H + h) * nsplit + z;
+    float* pa = part_acc + pidx * R;
+#pragma unroll
+    for (int j = 0; j < OT; ++j) {
+      const int t = j * 4 + wave, r = t * 16 + kq * 4;
+      if (t < rt && r < R) *reinterpret_cast<f32x4_t*>(pa + r) = o[j];
+    }
+    if (wave == 0 && kq == 0) {
       part_ml[pidx * 2] = m * LM_LN2;
       part_ml[pidx * 2 + 1] = lt;
     }
@@ -776,7 +1007,43 @@ static int launch_latent_attention(const void* q, void* out, const void* plane,
   return za_launch_status();
 }
 
-template <int WS, int RT, int NW>
+// The same for up to 64 ranges, a workgroup a row: the first wave turns the ranges' maxima
+// and sums into weights, then every thread adds up its elements over the ranges, in the
+// order of the ranges, with loads that do not wait for each other.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_combine_wide_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                           T* __restrict__ out, int R, int nsplit, const float* __restrict__ sink,
+                           int H) {
+  __shared__ float wz[64];
+  __shared__ float tot;
+  const size_t row = blockIdx.x;  // token * H + head
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    float mz = -INFINITY, lz = 0.f;
+    if (tid < nsplit) {
+      mz = part_ml[(row * nsplit + tid) * 2];
+      lz = part_ml[(row * nsplit + tid) * 2 + 1];
+    }
+    const float mx = wave_max(mz);
+    const float w = mz > -INFINITY ? expf(mz - mx) : 0.f;
+    float total = wave_sum(lz * w);
+    if (sink && mx > -INFINITY) total += expf(sink[row % H] - mx);
+    wz[tid] = w;
+    if (tid == 0) tot = total;
+  }
+  __syncthreads();
+  const float inv = tot > 0.f ? 1.0f / tot : 0.f;
+  for (int dd = tid; dd < R; dd += 256) {
+    const float* pa = part_acc + row * nsplit * R + dd;
+    float acc = 0.f;
+#pragma unroll 4
+    for (int z = 0; z < nsplit; ++z) acc = fmaf(pa[(size_t)z * R], wz[z], acc);
+    out[row * R + dd] = from_f32<T>(acc * inv);
+  }
+}
+
+template <int WS, int RT, bool DECODE>
 static int launch_latent_mfma(const void* q, void* out, const void* plane, long long page_stride,
                               const int* block_table, int bt_stride, const int* positions,
                               const int* wi_seq, const int* wi_row0, const int* wi_count,
@@ -784,8 +1051,9 @@ static int launch_latent_mfma(const void* q, void* out, const void* plane, long 
                               int page_size, float scale, int keys_per_split, int nsplit,
                               const float* sink, hipStream_t stream) {
   const int ws = (W + 31) / 32, rt = (R + 15) / 16;
-  const size_t shmem = ((size_t)LM_KT * (ws * 32 + 8) + (size_t)rt * 16 * LM_VS) * sizeof(bf16_t);
-  auto kernel = latent_attention_mfma_kernel<WS, RT, NW>;
+  const size_t shmem = ((size_t)LM_KT * (ws * 32 + 8) + (size_t)8 * lm_vp(rt) * LM_VS) * sizeof(bf16_t) +
+                       (DECODE ? 4 * 64 * 8 * sizeof(float) : 0);
+  auto kernel = DECODE ? latent_decode_mfma_kernel<WS, RT> : latent_attention_mfma_kernel<WS, RT>;
   static size_t allowed = 0;
   if (shmem > allowed) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel,
@@ -793,18 +1061,25 @@ static int launch_latent_mfma(const void* q, void* out, const void* plane, long 
     if (e != hipSuccess) return (int)e;
     allowed = shmem;
   }
-  const int HC = H < NW * 16 ? H : NW * 16;
-  dim3 grid(n_items, (H + HC - 1) / HC, nsplit), block(NW * 64);
+  int shift = -1;
+  if ((page_size & (page_size - 1)) == 0) {
+    shift = 0;
+    while ((1 << shift) < page_size) ++shift;
+  }
+  const int most = DECODE ? 16 : 64;
+  const int HC = H < most ? H : most;
+  dim3 grid(n_items, (H + HC - 1) / HC, nsplit), block(LM_NT);
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const bf16_t*)q, (bf16_t*)out,
                      (const bf16_t*)plane, page_stride, block_table, bt_stride, positions, wi_seq,
-                     wi_row0, wi_count, part_acc, part_ml, H, HC, W, R, page_size,
+                     wi_row0, wi_count, part_acc, part_ml, H, HC, W, R, page_size, shift,
                      scale * LM_LOG2E, keys_per_split, nsplit, sink);
   return za_launch_status();
 }
 
 // The matrix-core form: bfloat16, `width` and `kv_rank` multiples of 8.  `waves`: 4 (work
-// items of at most 64 / min(heads, 64) tokens) or 1 (single tokens, as a step that only
-// decodes has; heads in chunks of 16).  Arguments otherwise as za_latent_attention.
+// items of at most 64 / min(heads, 64) tokens, 16 rows a wave) or 1 (single tokens, as a
+// step that only decodes has: heads in chunks of 16 whose rows the four waves share).
+// Arguments otherwise as za_latent_attention.
 extern "C" int za_latent_attention_mfma(const void* q, void* out, const void* plane,
                                         long long page_stride, const int* block_table,
                                         int bt_stride, const int* positions, const int* wi_seq,
@@ -830,18 +1105,23 @@ extern "C" int za_latent_attention_mfma(const void* q, void* out, const void* pl
       n_items, part_acc, part_ml, heads, width, kv_rank, page_size, scale, keys_per_split,      \
       nsplit, sink, stream
   if (ws <= 6 && rt <= 8)
-    rc = waves == 4 ? launch_latent_mfma<6, 8, 4>(ZA_LM_ARGS) : launch_latent_mfma<6, 8, 1>(ZA_LM_ARGS);
+    rc = waves == 4 ? launch_latent_mfma<6, 8, false>(ZA_LM_ARGS)
+                    : launch_latent_mfma<6, 8, true>(ZA_LM_ARGS);
   else if (ws <= 10 && rt <= 16)
-    rc = waves == 4 ? launch_latent_mfma<10, 16, 4>(ZA_LM_ARGS)
-                    : launch_latent_mfma<10, 16, 1>(ZA_LM_ARGS);
+    rc = waves == 4 ? launch_latent_mfma<10, 16, false>(ZA_LM_ARGS)
+                    : launch_latent_mfma<10, 16, true>(ZA_LM_ARGS);
   else
-    rc = waves == 4 ? launch_latent_mfma<18, 32, 4>(ZA_LM_ARGS)
-                    : launch_latent_mfma<18, 32, 1>(ZA_LM_ARGS);
+    rc = waves == 4 ? launch_latent_mfma<18, 32, false>(ZA_LM_ARGS)
+                    : launch_latent_mfma<18, 32, true>(ZA_LM_ARGS);
 #undef ZA_LM_ARGS
   if (rc != 0 || nsplit == 1) return rc;
-  dim3 grid((unsigned)((size_t)n_tokens * heads)), block(64);
-  hipLaunchKernelGGL((latent_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc, part_ml,
-                     (bf16_t*)out, kv_rank, nsplit, 0, sink, heads);
+  dim3 grid((unsigned)((size_t)n_tokens * heads));
+  if (nsplit <= 64)
+    hipLaunchKernelGGL((latent_combine_wide_kernel<bf16_t>), grid, dim3(256), 0, stream, part_acc,
+                       part_ml, (bf16_t*)out, kv_rank, nsplit, sink, heads);
+  else
+    hipLaunchKernelGGL((latent_combine_kernel<bf16_t>), grid, dim3(64), 0, stream, part_acc,
+                       part_ml, (bf16_t*)out, kv_rank, nsplit, 0, sink, heads);
   return za_launch_status();
 }
 
