@@ -677,7 +677,9 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
   bf16_t* Vt = Ks + LM_KT * KS;                     // [8 * VP][LM_VS]
   const int VP = lm_vp(rt);
 
-  const int item = blockIdx.x, z = blockIdx.z;
+  // the last items first: within a request the later an item, the more keys it has, and
+  // workgroups start in the order of their numbers, so the long ones do not start last
+  const int item = gridDim.x - 1 - blockIdx.x, z = blockIdx.z;
   const int h0 = blockIdx.y * HC;
   const int G = min(HC, H - h0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
