@@ -164,6 +164,36 @@ def test_every_mechanism_counts():
         assert changed(**kw) > 0.02, name
 
 
+# ------------------------------- sizes that are multiples of nothing the kernels like
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_awkward_sizes(dtype):
+    cfg = gu.config([
+        gu.layer("latent_attention", gu.latent(heads=3, dim=12, vdim=20, kv_rank=28, q_rank=12,
+                                               rot_dim=6, base=77.0),
+                 gu.moe(ff=20, experts=7, identity=2, top=3, groups=(3, 2), shared=12)),
+        gu.layer("latent_attention_2", gu.plain_latent(heads=7, dim=10, vdim=6, kv_rank=18, q_rank=14),
+                 gu.moe(ff=12, experts=2, identity=0, top=1, shared=0)),
+        gu.layer("latent_attention", gu.latent(heads=70, dim=8, vdim=8, kv_rank=16, q_rank=24,
+                                               rot_dim=8), None),
+    ], width=36, vocab=53, side=6, softcap=9.0, mult=0.7)
+    model, tensors = build(cfg, seed=17, dtype=dtype)
+    lengths = [50, 3, 21]
+    prompts = [gu.tokens(n, cfg["vocab"], 30 + i) for i, n in enumerate(lengths)]
+    want = plain_logits(cfg, tensors, prompts)
+    base = None
+    for name, schedule in (("whole", eu.whole(lengths)),
+                           ("portions", eu.changing_portions(lengths, seed=2)),
+                           ("mixed", eu.mixed(lengths, seed=3, max_live=3, decode_tail=8))):
+        got = eu.run_schedule(runner_for(model, page_size=8, tokens=128, slots=3), prompts, schedule)
+        if dtype == "float32":
+            for g, w in zip(got, want):
+                assert worst(g, w) < F32_BOUND, name
+        else:
+            assert_bfloat16_close(torch.cat(got), torch.cat(want), name)
+            base = base or got
+            assert_bfloat16_same_run(torch.cat(got), torch.cat(base), name)
+
+
 # -------------------------------------------------------- schedules of whole models
 LENGTHS = [150, 37, 9, 1, 75, 130, 2]
 
@@ -482,18 +512,46 @@ def test_generation_bfloat16_runs_through_graphs():
     assert good >= 0.9 * total, (good, total)
 
 
-def test_command_line_generates(tmp_path):
+def test_trace_replay_and_command_line(tmp_path):
     import json
+    import os
     import subprocess
     import sys
-    import os
+    import numpy as np
     cfg = gu.TINY_ALL
-    d, _ = gu.folder(cfg, seed=8)
+    d, tensors = gu.folder(cfg, seed=8)
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = subprocess.run([sys.executable, "-m", "zig_ai_amd", "-m", d, "--prompt-ids", "5 17 3 100",
-                          "-n", "6", "--temperature", "0", "--dtype", "float32"],
-                         cwd=root, capture_output=True, text=True, timeout=600)
+    prompt, other = gu.tokens(40, cfg["vocab"], 3), gu.tokens(11, cfg["vocab"], 4)
+    want = plain.forward(cfg, tensors, prompt).float()
+    want_other = plain.forward(cfg, tensors, other).float()
+    # portions of one request beside another's, single tokens, a step in which nothing is asked
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": prompt[:25], "want": [3, 24]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": prompt[25:27], "want": []},
+                                     {"id": "b", "tokens": other[:10], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": other[10:], "want": [0]},
+                                     {"id": "a", "tokens": prompt[27:], "want": [12]}], "end": ["a", "b"]}]
+    out = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d,
+                          "--dtype", "float32", "--out", str(tmp_path), "--max-tokens", "128"],
+                         input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                         capture_output=True, timeout=600)
     assert out.returncode == 0, out.stderr[-2000:]
+    assert [l for l in out.stdout.split("\n") if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    first = torch.from_numpy(np.fromfile(tmp_path / "0.f32", dtype="<f4").reshape(2, -1))
+    last = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(2, -1))
+    assert not (tmp_path / "1.f32").exists()
+    assert worst(torch.cat([first, last[1:]]), want[[3, 24, 39]]) < F32_BOUND
+    assert worst(last[:1], want_other[[10]]) < F32_BOUND
+    gen = subprocess.run([sys.executable, "-m", "zig_ai_amd", "--model", d, "--dtype", "float32",
+                          "--prompt-ids", ",".join(map(str, prompt[:9])), "-n", "5",
+                          "--temperature", "0", "--json"], cwd=root, text=True, capture_output=True,
+                         timeout=600)
+    assert gen.returncode == 0, gen.stderr[-2000:]
+    outputs = json.loads(gen.stdout.strip().split("\n")[-1])["outputs"]
+    assert len(outputs) == 1 and len(outputs[0]) == 5
+    logits = plain.forward(cfg, tensors, prompt[:9] + outputs[0])
+    for j, tok in enumerate(outputs[0]):
+        row = logits[9 + j - 1]
+        assert float(row.max() - row[tok]) <= 1e-3 * float(row.abs().max()), (j, tok)
 
 
 # ------------------------------------------------------------------ kernels alone
