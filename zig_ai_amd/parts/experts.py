@@ -187,7 +187,12 @@ class RoutedExperts(FeedForward):
                                      out_dtype=torch.float32)
         shared = None
         if self.shared_gate_up is not None:
-            s = ops.gated_unit(ops.linear(x, self.shared_gate_up, tune=tune), self.activation)
+            if x.dtype == torch.bfloat16 and self.shared_gate_up.dtype == torch.bfloat16 \
+                    and T <= 16 and x.shape[1] <= 8192:
+                # a decode batch: the gate is applied to the projection's accumulators
+                s = ops.linear_swiglu(x, self.shared_gate_up, self.activation)
+            else:
+                s = ops.gated_unit(ops.linear(x, self.shared_gate_up, tune=tune), self.activation)
             shared = ops.linear(s, self.shared_down, out_dtype=torch.float32, tune=tune)
         return ops.experts_combine(out, chosen, weight, x, self.experts, shared,
                                    logits if self.shared_gated else None, self.outputs)
