@@ -19,7 +19,9 @@
 //   latent_attention   the attention itself: causal, streaming softmax in 32-bit with a sink
 //                      a head, any mix of prompt portions and single tokens in one launch,
 //                      contexts optionally cut into ranges (latent_combine merges them)
-//   latent_attention_mfma   the same on the matrix cores (bfloat16)
+//   latent_attention_mfma   the same on the matrix cores (bfloat16, 16-byte pieces): four waves
+//                      of 16 rows each for prompt portions and mixed steps
+//   latent_decode_mfma      steps that only decode: four waves share 16 rows
 // Rotation: adjacent pairs (2i, 2i + 1) or halves (i, i + dims/2) of the first `rot_dims`
 // elements, angle = position * inv_freq[i] in 32-bit.
 #include <math.h>

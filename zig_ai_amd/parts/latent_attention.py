@@ -15,7 +15,10 @@ Per token, with ``h`` the mixer's input:
 Only ``[c | rot(k_r)]`` is cached, one plane of ``kv_rank + rotated_dim`` elements a token, and
 keys and values are never formed: ``Wuk_i^T q_i,n`` is taken instead (the score against ``c``
 is the same number) and ``Wuv_i`` is applied to ``sum_j p_j c_j``, so the attention kernel sees
-one key/value head whose value is a prefix of its key (``csrc/latent.hip``).
+one key/value head whose value is a prefix of its key (``csrc/latent.hip``).  bfloat16 rows of
+16-byte pieces run on the matrix cores (work items of 64 rows; a step that only decodes takes the
+kernel whose four waves share 16 rows, its contexts cut into ranges), everything else the
+general kernel.
 
 All sizes and constants come from ``params``: ``hidden_size, num_heads, head_dim,
 rotated_dim`` (0: no positions), ``value_dim, kv_rank, q_rank, softmax_scale`` (None:
