@@ -39,7 +39,7 @@ import numpy as np
 import torch
 
 from ..kernels import host
-from ..parts.base import PagedNeed, StateNeed
+from ..parts.base import PagedNeed, PagedStateNeed, StateNeed
 from .pages import Pool, raise_for
 
 FREED = -1   # block-table entry of a page that was given back (behind the window)
@@ -128,6 +128,10 @@ class CacheManager:
         for cid, need in needs.items():
             if need is None:
                 continue
+            if isinstance(need, PagedStateNeed):
+                # both: its pages are grouped like any paged need's, its state lies in the slot
+                state_entries.append((cid, need.state))
+                need = need.paged
             if isinstance(need, PagedNeed):
                 if not need.planes or any(h <= 0 or w <= 0 for h, w in need.planes):
                     raise ValueError(f"cache entry {cid!r}: a paged need has planes of positive "
@@ -212,6 +216,8 @@ class CacheManager:
         the same number of pages when ``num_pages`` is a single number)."""
         total = 0
         for need in needs.values():
+            if isinstance(need, PagedStateNeed):
+                need = need.paged
             if isinstance(need, PagedNeed):
                 size = torch.empty((), dtype=need.dtype or run_dtype).element_size()
                 total += need.elements_per_token() * page_size * size
@@ -219,19 +225,20 @@ class CacheManager:
 
     # ------------------------------------------------------------------ views
     def view(self, cache_id, writes: bool = True) -> CacheView:
+        st = None
+        if cache_id in self._state_layout and self.slot_memory is not None:
+            # A window of every slot's row: contiguous within a slot, slots spaced by
+            # the whole row.
+            off, nbytes, shape, dtype = self._state_layout[cache_id]
+            st = self.slot_memory[:, off:off + nbytes].view(dtype).unflatten(1, shape)
         if cache_id in self._group_of:
+            # (an entry that needs pages and a state has both in its view)
             grp = self.groups[self._group_of[cache_id]]
             layer = grp.layer_of(cache_id)
             kv = grp.kv[layer] if grp.kv is not None else None
             return CacheView("paged", group=grp.index, kv=kv, planes=grp.plane_views(layer),
-                             writes=writes)
+                             state=st, writes=writes)
         if cache_id in self._state_layout:
-            off, nbytes, shape, dtype = self._state_layout[cache_id]
-            st = None
-            if self.slot_memory is not None:
-                # A window of every slot's row: contiguous within a slot, slots spaced by
-                # the whole row.
-                st = self.slot_memory[:, off:off + nbytes].view(dtype).unflatten(1, shape)
             return CacheView("state", state=st, writes=writes)
         return CacheView("none", writes=writes)
 

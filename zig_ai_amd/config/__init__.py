@@ -18,6 +18,7 @@ from .lfm2 import Lfm2Config, feed_forward_width  # noqa: F401
 from .rudilix import RudilixConfig  # noqa: F401
 from .ranesun import RanesunConfig  # noqa: F401
 from .gemodra import GemodraConfig  # noqa: F401
+from .nopozen import NopozenConfig  # noqa: F401
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -70,3 +71,4 @@ register_architecture("Lfm2ForCausalLM", Lfm2Config)
 register_architecture("Rudilix", RudilixConfig)
 register_architecture("Ranesun", RanesunConfig)
 register_architecture("Gemodra", GemodraConfig)
+register_architecture("Nopozen", NopozenConfig)

@@ -243,6 +243,50 @@ extern "C" int za_gated_unit(const void* gu, void* out, int dtype, int n_tokens,
   return za_launch_status();
 }
 
+// A feed-forward's activation on its own, element by element, in 32-bit:
+//   act 0: the square of relu, max(x, 0)^2
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+activate_kernel(const T* __restrict__ in, T* __restrict__ out, size_t total, int act) {
+  const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  if (idx >= total) return;
+  if (VEC == 8) {
+    float x[8], o[8];
+    load8<T>(in + idx, x);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float r = fmaxf(x[k], 0.f);
+      o[k] = r * r;
+    }
+    store8<T>(out + idx, o);
+  } else {
+    const float r = fmaxf(to_f32<T>(in[idx]), 0.f);
+    out[idx] = from_f32<T>(r * r);
+  }
+}
+
+extern "C" int za_activate(const void* in, void* out, int dtype, long long n, int act,
+                           hipStream_t stream) {
+  if (n == 0) return 0;
+  if (n < 0 || !in || !out || act != 0) return ZA_ERR_ARG;
+  const size_t total = (size_t)n;
+  const bool vec = total % 8 == 0;
+  const size_t threads = vec ? total / 8 : total;
+  dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+#define ZA_ACT(T, V)                                                                         \
+  hipLaunchKernelGGL((activate_kernel<T, V>), grid, block, 0, stream, (const T*)in, (T*)out, \
+                     total, act)
+  if (dtype == 0) {
+    if (vec) ZA_ACT(float, 8); else ZA_ACT(float, 1);
+  } else if (dtype == 1) {
+    if (vec) ZA_ACT(bf16_t, 8); else ZA_ACT(bf16_t, 1);
+  } else {
+    return ZA_ERR_UNSUPPORTED;
+  }
+#undef ZA_ACT
+  return za_launch_status();
+}
+
 // x <- x * s, 32-bit, in place (an output head's constant factor on its logits).
 __global__ void __launch_bounds__(256) scale_kernel(float* __restrict__ x, float s, size_t n) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -2,7 +2,8 @@
 // prompt portions and single decoded tokens in one launch.
 //
 //   s[t,h,j] = (q[t,h] . k[j,kv(h)]) * scale,  kv(h) = h / (nh / nkv)
-//   keys j <= position(t) only, and j > position(t) - window when window > 0
+//   keys j <= position(t) only, and j > position(t) - window when window > 0, and
+//   floor(j / chunk) = floor(position(t) / chunk) when chunk > 0 (the general kernel)
 //   softmax over j in 32-bit, streaming: running maximum m and sum l, the
 //   accumulator rescaled by exp(m_old - m_new) when the maximum moves
 //   o[t,h]   = sum_j p[j] v[j,kv(h)] / l
@@ -95,11 +96,14 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
                        float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv,
                        int d, int page_size, float scale, int window, int keys_per_split,
                        int nsplit, int dv, const T* __restrict__ gate, int gate_stride,
-                       int gate_col, float out_scale, ScoreExtras ex) {
+                       int gate_col, float out_scale, ScoreExtras ex, int chunk, int gate_elem) {
   // `dv`: width of a value (keys and queries have `d`); a page holds the keys of all
   // heads, [kv_head][offset][d], then the values turned round, [kv_head][dv][offset].
   // `gate`: when given, head h of token t is multiplied by
-  // sigmoid(gate[t * gate_stride + gate_col + h]) * out_scale.
+  // sigmoid(gate[t * gate_stride + gate_col + h]) * out_scale; with `gate_elem` every
+  // element dd of it by its own sigmoid(gate[t * gate_stride + gate_col + h * dv + dd]).
+  // `chunk` > 0: positions are counted in chunks of that many from the sequence's start,
+  // and a query sees the keys of its own chunk only.
   extern __shared__ float smem[];
   const int ldk = d + 1, ldv = dv + 1;
   const size_t page_elems = (size_t)nkv * page_size * (d + dv);
@@ -121,7 +125,8 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
 
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
-  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  if (chunk > 0 && (pos_first / chunk) * chunk > lo) lo = (pos_first / chunk) * chunk;
   const int hi = pos_last;  // inclusive
   int range_lo = z * keys_per_split;
   int range_hi = range_lo + keys_per_split - 1;
@@ -192,6 +197,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
         const int kp = tile0 + lane;
         bool valid = lane < KT && kp <= pos && kp <= range_hi && kp >= lo;
         if (window > 0 && kp <= pos - window) valid = false;
+        if (chunk > 0 && kp < (pos / chunk) * chunk) valid = false;
         float s = -INFINITY;
         if (lane < KT) {
           const float* qr = Qs + r * d;
@@ -237,7 +243,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
         if (ex.sink) l[lr] += expf(ex.sink[h] - m[lr]);
         const float inv = l[lr] > 0.f ? 1.0f / l[lr] : 0.f;
         float mult = 1.0f;
-        if (gate) {
+        if (gate && !gate_elem) {
           const float gl = to_f32<T>(gate[(size_t)tok * gate_stride + gate_col + h]);
           mult = out_scale / (1.0f + expf(-gl));
         }
@@ -245,7 +251,14 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
 #pragma unroll
         for (int c = 0; c < AT_DPL; ++c) {
           const int dd = lane + 64 * c;
-          if (dd < dv) o[dd] = from_f32<T>(gate ? acc[lr][c] * inv * mult : acc[lr][c] * inv);
+          if (dd < dv) {
+            if (gate && gate_elem) {
+              const float gl =
+                  to_f32<T>(gate[(size_t)tok * gate_stride + gate_col + (size_t)h * dv + dd]);
+              mult = out_scale / (1.0f + expf(-gl));
+            }
+            o[dd] = from_f32<T>(gate ? acc[lr][c] * inv * mult : acc[lr][c] * inv);
+          }
         }
       } else {
         const size_t pidx = ((size_t)tok * nh + h) * nsplit + z;
@@ -1144,7 +1157,7 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
                             float* part_ml, int nh, int nkv, int d, int page_size, float scale,
                             int window, int keys_per_split, int nsplit, int dv, const void* gate,
                             int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                            hipStream_t stream) {
+                            int chunk, int gate_elem, hipStream_t stream) {
   const size_t shmem = ((size_t)KT * (d + 1) + (size_t)KT * (dv + 1) + (size_t)AT_MAX_ROWS * d +
                         AT_WAVES * 64) * sizeof(float);
   auto kernel = paged_attention_kernel<T, KT>;
@@ -1159,7 +1172,7 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)kv,
                      block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, part_acc,
                      part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv,
-                     (const T*)gate, gate_stride, gate_col, out_scale, ex);
+                     (const T*)gate, gate_stride, gate_col, out_scale, ex, chunk, gate_elem);
   return za_launch_status();
 }
 
@@ -1168,33 +1181,52 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_gate_kernel(T* __restrict__ out, const T* __restrict__ gate, int gate_stride, int gate_col,
-                 int nh, int dv, float out_scale, size_t total) {
+                 int nh, int dv, float out_scale, size_t total, int gate_elem) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t row = idx / dv;             // token * nh + head
   const size_t tok = row / nh;
   const int h = (int)(row % nh);
-  const float gl = to_f32<T>(gate[tok * gate_stride + gate_col + h]);
+  // (`gate_elem`: a gate an element, laid out head by head like the output itself)
+  const size_t col = gate_elem ? (size_t)h * dv + idx % dv : (size_t)h;
+  const float gl = to_f32<T>(gate[tok * gate_stride + gate_col + col]);
   out[idx] = from_f32<T>(to_f32<T>(out[idx]) * (out_scale / (1.0f + expf(-gl))));
 }
 
-extern "C" int za_head_gate(void* out, const void* gate, int dtype, int gate_stride, int gate_col,
-                            int n_tokens, int nh, int dv, float out_scale, hipStream_t stream) {
+static int head_gate_any(void* out, const void* gate, int dtype, int gate_stride, int gate_col,
+                         int n_tokens, int nh, int dv, float out_scale, int gate_elem,
+                         hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (n_tokens < 0 || nh <= 0 || dv <= 0 || !out || !gate || gate_col < 0 ||
-      gate_col + nh > gate_stride)
+      gate_col + (gate_elem ? nh * dv : nh) > gate_stride)
     return ZA_ERR_ARG;
   const size_t total = (size_t)n_tokens * nh * dv;
   dim3 grid((unsigned)((total + 255) / 256)), block(256);
   if (dtype == 0)
     hipLaunchKernelGGL((head_gate_kernel<float>), grid, block, 0, stream, (float*)out,
-                       (const float*)gate, gate_stride, gate_col, nh, dv, out_scale, total);
+                       (const float*)gate, gate_stride, gate_col, nh, dv, out_scale, total,
+                       gate_elem);
   else if (dtype == 1)
     hipLaunchKernelGGL((head_gate_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)out,
-                       (const bf16_t*)gate, gate_stride, gate_col, nh, dv, out_scale, total);
+                       (const bf16_t*)gate, gate_stride, gate_col, nh, dv, out_scale, total,
+                       gate_elem);
   else
     return ZA_ERR_UNSUPPORTED;
   return za_launch_status();
+}
+
+extern "C" int za_head_gate(void* out, const void* gate, int dtype, int gate_stride, int gate_col,
+                            int n_tokens, int nh, int dv, float out_scale, hipStream_t stream) {
+  return head_gate_any(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, 0,
+                       stream);
+}
+
+// The same with a gate an element: gate[t * gate_stride + gate_col + h * dv + dd].
+extern "C" int za_element_gate(void* out, const void* gate, int dtype, int gate_stride,
+                               int gate_col, int n_tokens, int nh, int dv, float out_scale,
+                               hipStream_t stream) {
+  return head_gate_any(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, 1,
+                       stream);
 }
 
 static int paged_attention_any(const void* q, void* out, const void* kv, const int* block_table,
@@ -1204,7 +1236,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
                                int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                               hipStream_t stream);
+                               hipStream_t stream, int chunk = 0, int gate_elem = 0);
 
 // dtype codes: 0 = float32, 1 = bfloat16
 extern "C" int za_paged_attention(const void* q, void* out, const void* kv, const int* block_table,
@@ -1265,8 +1297,9 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
                                int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                               hipStream_t stream) {
+                               hipStream_t stream, int chunk, int gate_elem) {
   if (n_items == 0 || n_tokens == 0) return 0;
+  if (chunk < 0) return ZA_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || d <= 0 || page_size <= 0 ||
       bt_stride <= 0 || nsplit < 1 || !q || !out || !kv || !block_table || !positions ||
       !wi_seq || !wi_row0 || !wi_count)
@@ -1279,7 +1312,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
 #define ZA_AT_ARGS                                                                            \
   q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, part_acc, \
       part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv, gate,         \
-      gate_stride, gate_col, out_scale, ex, stream
+      gate_stride, gate_col, out_scale, ex, chunk, gate_elem, stream
   const bool small = d <= 128 && dv <= 128;
   if (dtype == 0) {
     rc = small ? launch_attention<float, 64>(ZA_AT_ARGS) : launch_attention<float, 32>(ZA_AT_ARGS);
@@ -1300,7 +1333,29 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                        part_ml, (bf16_t*)out, dv, nsplit, 0, ex.sink, nh);
   rc = za_launch_status();
   if (rc != 0 || !gate) return rc;
-  return za_head_gate(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, stream);
+  return head_gate_any(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale,
+                       gate_elem, stream);
+}
+
+// Everything the general kernel knows, at once: values of width `dv`, an output gate a head
+// or (`gate_elem`) an element, what `ScoreExtras` describes, a window and chunks.
+extern "C" int za_paged_attention_general(
+    const void* q, void* out, const void* kv, const int* block_table, int bt_stride,
+    const int* positions, const int* wi_seq, const int* wi_row0, const int* wi_count, int n_items,
+    int n_tokens, float* part_acc, float* part_ml, int dtype, int nh, int nkv, int d, int dv,
+    int page_size, float scale, int window, int chunk, int keys_per_split, int nsplit,
+    const void* gate, int gate_stride, int gate_col, int gate_elem, float out_scale, float softcap,
+    const float* sink, float qt_coef, int qt_every, hipStream_t stream) {
+  if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D || softcap < 0.f || qt_every < 0 || chunk < 0)
+    return ZA_ERR_UNSUPPORTED;
+  if (gate && (gate_col < 0 || gate_col + (gate_elem ? nh * dv : nh) > gate_stride))
+    return ZA_ERR_ARG;
+  return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                             wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
+                             page_size, scale, window, keys_per_split, nsplit, dv, gate,
+                             gate_stride, gate_col, out_scale,
+                             ScoreExtras{softcap, sink, qt_coef, qt_every}, stream, chunk,
+                             gate_elem);
 }
 
 template <int D, int KT, bool SHAPED>

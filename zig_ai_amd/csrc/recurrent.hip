@@ -3,7 +3,7 @@
 // recurrence is 32-bit: the state, decays, step sizes, gates and unit norms.
 //
 // 1. causal_conv_silu: a depth-wise causal convolution over a request's own inputs
-//    followed by silu,
+//    followed by silu (or, through za_causal_conv, by nothing),
 //      y[t, c] = silu(bias[c] + sum_j taps[c, j] * x[t - (L - 1 - j), c]),
 //    the L - 1 inputs before a portion coming from the request's state slot, which
 //    afterwards holds the portion's last L - 1 inputs.
@@ -50,14 +50,15 @@ __device__ __forceinline__ float softplus_f(float x) {
 // grid.x: blocks of 256 channels; grid.y: first the blocks of `tokens_per_block`
 // tokens (bodies: tokens whose L - 1 predecessors lie in the same portion), then one
 // block per request (heads: the first L - 1 tokens of its portion and the state).
-template <typename T>
+// `act`: 1 silu, 0 none.  `TO`: what is stored (the state keeps 32-bit inputs either way).
+template <typename T, typename TO>
 __global__ void __launch_bounds__(256)
 causal_conv_silu_kernel(const T* __restrict__ x, int x_stride, int col0,
                         const float* __restrict__ taps, const float* __restrict__ bias,
                         float* __restrict__ state, long long slot_stride,
                         const int* __restrict__ token_seq, const int* __restrict__ seq_start,
-                        const int* __restrict__ slot_id, float* __restrict__ out, int n_tokens,
-                        int C, int L, int body_blocks, int tokens_per_block) {
+                        const int* __restrict__ slot_id, TO* __restrict__ out, int n_tokens,
+                        int C, int L, int body_blocks, int tokens_per_block, int act) {
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= C) return;
   float w[RC_MAX_TAPS];
@@ -87,7 +88,7 @@ causal_conv_silu_kernel(const T* __restrict__ x, int x_stride, int col0,
       for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
         if (j < L - 1) acc = fmaf(w[j], before[j], acc);
       acc = fmaf(w[L - 1], xi, acc);
-      out[(size_t)t * C + c] = silu_f(acc);
+      out[(size_t)t * C + c] = from_f32<TO>(act ? silu_f(acc) : acc);
 #pragma unroll
       for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
         if (j < L - 2) before[j] = before[j + 1];
@@ -109,7 +110,7 @@ causal_conv_silu_kernel(const T* __restrict__ x, int x_stride, int col0,
     for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
       if (j < L - 1) acc = fmaf(w[j], hist[j], acc);
     acc = fmaf(w[L - 1], xi, acc);
-    out[(size_t)(start + i) * C + c] = silu_f(acc);
+    out[(size_t)(start + i) * C + c] = from_f32<TO>(act ? silu_f(acc) : acc);
 #pragma unroll
     for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
       if (j < L - 2) hist[j] = hist[j + 1];
@@ -126,31 +127,41 @@ causal_conv_silu_kernel(const T* __restrict__ x, int x_stride, int col0,
     if (j < L - 1) st[j] = hist[j];
 }
 
-extern "C" int za_causal_conv_silu(const void* x, int dtype, int x_stride, int col0,
-                                   const float* taps, const float* bias, float* state,
-                                   long long slot_stride, const int* token_seq,
-                                   const int* seq_start, const int* slot_id, float* out,
-                                   int n_tokens, int n_seqs, int C, int L, hipStream_t stream) {
+// `act`: 1 silu, 0 none; `out_dtype`: 0 the result as 32-bit floats, 1 as bfloat16.
+extern "C" int za_causal_conv(const void* x, int dtype, int x_stride, int col0, const float* taps,
+                              const float* bias, float* state, long long slot_stride,
+                              const int* token_seq, const int* seq_start, const int* slot_id,
+                              void* out, int out_dtype, int act, int n_tokens, int n_seqs, int C,
+                              int L, hipStream_t stream) {
   if (n_tokens == 0 || n_seqs == 0) return 0;
   if (n_tokens < 0 || n_seqs < 0 || C <= 0 || !x || !taps || !state || !token_seq || !seq_start ||
-      !slot_id || !out || col0 < 0 || col0 + C > x_stride || slot_stride < (long long)C * (L - 1))
+      !slot_id || !out || col0 < 0 || col0 + C > x_stride || slot_stride < (long long)C * (L - 1) ||
+      act < 0 || act > 1)
     return ZA_ERR_ARG;
   if (L < 1 || L > RC_MAX_TAPS) return ZA_ERR_UNSUPPORTED;
   const int tpb = 16;
   // (single tokens with a state to read: heads only)
   const int body = (n_tokens > n_seqs || L == 1) ? (n_tokens + tpb - 1) / tpb : 0;
   dim3 grid((C + 255) / 256, body + n_seqs), block(256);
-  if (dtype == 0)
-    hipLaunchKernelGGL((causal_conv_silu_kernel<float>), grid, block, 0, stream, (const float*)x,
-                       x_stride, col0, taps, bias, state, slot_stride, token_seq, seq_start,
-                       slot_id, out, n_tokens, C, L, body, tpb);
-  else if (dtype == 1)
-    hipLaunchKernelGGL((causal_conv_silu_kernel<bf16_t>), grid, block, 0, stream,
-                       (const bf16_t*)x, x_stride, col0, taps, bias, state, slot_stride, token_seq,
-                       seq_start, slot_id, out, n_tokens, C, L, body, tpb);
-  else
-    return ZA_ERR_UNSUPPORTED;
+#define ZA_CONV(T, TO)                                                                          \
+  hipLaunchKernelGGL((causal_conv_silu_kernel<T, TO>), grid, block, 0, stream, (const T*)x,      \
+                     x_stride, col0, taps, bias, state, slot_stride, token_seq, seq_start,       \
+                     slot_id, (TO*)out, n_tokens, C, L, body, tpb, act)
+  if (dtype == 0 && out_dtype == 0) ZA_CONV(float, float);
+  else if (dtype == 1 && out_dtype == 0) ZA_CONV(bf16_t, float);
+  else if (dtype == 1 && out_dtype == 1) ZA_CONV(bf16_t, bf16_t);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_CONV
   return za_launch_status();
+}
+
+extern "C" int za_causal_conv_silu(const void* x, int dtype, int x_stride, int col0,
+                                   const float* taps, const float* bias, float* state,
+                                   long long slot_stride, const int* token_seq,
+                                   const int* seq_start, const int* slot_id, float* out,
+                                   int n_tokens, int n_seqs, int C, int L, hipStream_t stream) {
+  return za_causal_conv(x, dtype, x_stride, col0, taps, bias, state, slot_stride, token_seq,
+                        seq_start, slot_id, out, 0, 1, n_tokens, n_seqs, C, L, stream);
 }
 
 // ------------------------------------------------------------------- recurrence
@@ -732,53 +743,67 @@ __global__ void __launch_bounds__(64)
 retention_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_col, int k_col,
                          int v_col, const int* __restrict__ positions,
                          const float* __restrict__ inv_freq, float* __restrict__ prep, int H,
-                         int dk, int dv, int rot, float k_scale) {
+                         int dk, int dv, int rot, float k_scale, int act) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const T* row = proj + (size_t)t * proj_stride;
   float* dst = prep + (size_t)t * (2 * H * dk + H * dv);
   const int pos = positions[t], half = rot / 2;
   for (int i = lane; i < dk; i += 64) {
-    const float q = to_f32<T>(row[q_col + h * dk + i]);
-    const float k = to_f32<T>(row[k_col + h * dk + i]);
+    // (`act` 1: silu on what the projection gave, before anything else)
+    float q = to_f32<T>(row[q_col + h * dk + i]);
+    float k = to_f32<T>(row[k_col + h * dk + i]);
+    if (act) { q = silu_f(q); k = silu_f(k); }
     float qo = q, ko = k;
     if (i < rot) {
       const bool low = i < half;
       const int j = low ? i : i - half, partner = low ? i + half : i - half;
       float cs, sn;
       rope_angle(pos, inv_freq[j], &cs, &sn);
-      const float qp = to_f32<T>(row[q_col + h * dk + partner]);
-      const float kp = to_f32<T>(row[k_col + h * dk + partner]);
+      float qp = to_f32<T>(row[q_col + h * dk + partner]);
+      float kp = to_f32<T>(row[k_col + h * dk + partner]);
+      if (act) { qp = silu_f(qp); kp = silu_f(kp); }
       qo = low ? rope_rotate_low(q, qp, cs, sn) : rope_rotate_high(q, qp, cs, sn);
       ko = low ? rope_rotate_low(k, kp, cs, sn) : rope_rotate_high(k, kp, cs, sn);
     }
     dst[h * dk + i] = qo;
     dst[H * dk + h * dk + i] = ko * k_scale;
   }
-  for (int i = lane; i < dv; i += 64)
-    dst[2 * H * dk + h * dv + i] = to_f32<T>(row[v_col + h * dv + i]);
+  for (int i = lane; i < dv; i += 64) {
+    const float v = to_f32<T>(row[v_col + h * dv + i]);
+    dst[2 * H * dk + h * dv + i] = act ? silu_f(v) : v;
+  }
+}
+
+extern "C" int za_retention_prepare_act(const void* proj, int dtype, int proj_stride, int q_col,
+                                    int k_col, int v_col, const int* positions,
+                                    const float* inv_freq, float* prep, int n_tokens, int H, int dk,
+                                    int dv, int rot, float k_scale, int act, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || H <= 0 || dk <= 0 || dv <= 0 || !proj || !positions || !prep || rot < 0 ||
+      rot > dk || rot % 2 || (rot > 0 && !inv_freq) || q_col < 0 || k_col < 0 || v_col < 0 ||
+      act < 0 || act > 1 || q_col + H * dk > proj_stride || k_col + H * dk > proj_stride ||
+      v_col + H * dv > proj_stride)
+    return ZA_ERR_ARG;
+  dim3 grid(n_tokens, H), block(64);
+  if (dtype == 0)
+    hipLaunchKernelGGL((retention_prepare_kernel<float>), grid, block, 0, stream,
+                       (const float*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
+                       prep, H, dk, dv, rot, k_scale, act);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((retention_prepare_kernel<bf16_t>), grid, block, 0, stream,
+                       (const bf16_t*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
+                       prep, H, dk, dv, rot, k_scale, act);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
 }
 
 extern "C" int za_retention_prepare(const void* proj, int dtype, int proj_stride, int q_col,
                                     int k_col, int v_col, const int* positions,
                                     const float* inv_freq, float* prep, int n_tokens, int H, int dk,
                                     int dv, int rot, float k_scale, hipStream_t stream) {
-  if (n_tokens == 0) return 0;
-  if (n_tokens < 0 || H <= 0 || dk <= 0 || dv <= 0 || !proj || !positions || !prep || rot < 0 ||
-      rot > dk || rot % 2 || (rot > 0 && !inv_freq) || q_col < 0 || k_col < 0 || v_col < 0 ||
-      q_col + H * dk > proj_stride || k_col + H * dk > proj_stride || v_col + H * dv > proj_stride)
-    return ZA_ERR_ARG;
-  dim3 grid(n_tokens, H), block(64);
-  if (dtype == 0)
-    hipLaunchKernelGGL((retention_prepare_kernel<float>), grid, block, 0, stream,
-                       (const float*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
-                       prep, H, dk, dv, rot, k_scale);
-  else if (dtype == 1)
-    hipLaunchKernelGGL((retention_prepare_kernel<bf16_t>), grid, block, 0, stream,
-                       (const bf16_t*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
-                       prep, H, dk, dv, rot, k_scale);
-  else
-    return ZA_ERR_UNSUPPORTED;
-  return za_launch_status();
+  return za_retention_prepare_act(proj, dtype, proj_stride, q_col, k_col, v_col, positions,
+                                  inv_freq, prep, n_tokens, H, dk, dv, rot, k_scale, 0, stream);
 }
 
 // ------------------------------------------------------------- gated group norm

@@ -122,6 +122,20 @@ _SIGNATURES = {
                                 c_int, c_int, c_void_p],
     ("activation", "za_gated_unit"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     ("activation", "za_scale"): [c_void_p, c_float, c_longlong, c_void_p],
+    ("recurrent", "za_causal_conv"): [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                      c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                      c_int, c_int, c_int, c_int, c_int, c_void_p],
+    ("recurrent", "za_retention_prepare_act"): [c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                                c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                                c_int, c_int, c_float, c_int, c_void_p],
+    ("activation", "za_activate"): [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
+    ("attention", "za_element_gate"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                       c_int, c_float, c_void_p],
+    ("attention", "za_paged_attention_general"): [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+        c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p, c_float,
+        c_int, c_void_p],
     ("recurrent", "za_retention_prepare"): [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
                                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                             c_float, c_void_p],
@@ -1441,6 +1455,22 @@ def gated_unit(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
     return out
 
 
+UNARY_ACTIVATIONS = {"relu2": 0}
+
+
+def activate(x: torch.Tensor, activation: str) -> torch.Tensor:
+    """A feed-forward's activation on its own, element by element, in 32-bit: ``relu2``, the
+    square of relu."""
+    if activation not in UNARY_ACTIVATIONS:
+        raise KernelError(f"activation must be one of {sorted(UNARY_ACTIVATIONS)}, got {activation!r}")
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    out = torch.empty_like(x)
+    rc = _fn("activation", "za_activate")(_ptr(x), _ptr(out), _code(x.dtype), x.numel(),
+                                          UNARY_ACTIVATIONS[activation], _stream())
+    _check(rc, "activate")
+    return out
+
+
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
     """``x *= factor`` for a 32-bit tensor, in place."""
     _need(x, "x", torch.float32)
@@ -1695,11 +1725,15 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
                           item_seq: torch.Tensor, item_row0: torch.Tensor, item_count: torch.Tensor,
                           n_items: int, scale: float, window: int = 0, keys_per_split: int = 0,
                           nsplit: int = 1, gate: Optional[torch.Tensor] = None, gate_col: int = 0,
-                          out_scale: float = 1.0) -> torch.Tensor:
+                          out_scale: float = 1.0, shape: Optional[ScoreShape] = None,
+                          chunk: int = 0, gate_element: bool = False) -> torch.Tensor:
     """``paged_attention`` for values of their own width: ``q [T, heads, head_dim]``, the
     cache as a plane of keys and a plane of values (see ``qk_norm_rope_kv_write_wide``);
     returns ``[T, heads, value_dim]``.  With ``gate [T, columns]`` head ``h`` of token ``t``
-    is multiplied by ``sigmoid(gate[t, gate_col + h]) * out_scale``."""
+    is multiplied by ``sigmoid(gate[t, gate_col + h]) * out_scale``, or with ``gate_element``
+    its element ``e`` by ``sigmoid(gate[t, gate_col + h * value_dim + e]) * out_scale``.
+    ``shape``: see ``ScoreShape``.  ``chunk > 0``: a query sees the keys ``j`` with
+    ``j // chunk == position // chunk`` only (chunks counted from the sequence's start)."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -1711,6 +1745,8 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
                           f"{ATTENTION_MAX_ROWS}")
     if d % 8 or dv % 8 or d > 256 or dv > 256:
         raise KernelError(f"head widths {d} and {dv} must be multiples of 8, at most 256")
+    if chunk < 0 or window < 0:
+        raise KernelError("window and chunk must not be negative")
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [requests, max_pages]")
@@ -1722,9 +1758,10 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
     gate_stride = 0
     if gate is not None:
         _need(gate, "gate", q.dtype)
-        if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + nh > gate.shape[1]:
+        columns = nh * dv if gate_element else nh
+        if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + columns > gate.shape[1]:
             raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
-                              f"{gate_col + nh} of {T} rows are needed")
+                              f"{gate_col + columns} of {T} rows are needed")
         gate_stride = gate.shape[1]
     out = torch.empty((T, nh, dv), dtype=q.dtype, device=q.device)
     part_acc = part_ml = None
@@ -1733,27 +1770,32 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
             raise KernelError("keys_per_split must be a positive multiple of 64")
         part_acc = torch.empty((T, nh, nsplit, dv), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
-    rc = _fn("attention", "za_paged_attention_gated")(
+    extras = shape.args(nh) if shape else (0.0, None, 0.0, 0)
+    rc = _fn("attention", "za_paged_attention_general")(
         _ptr(q), _ptr(out), _ptr(key_plane), _ptr(block_table), block_table.shape[1],
         _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
         _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, dv, page_size, float(scale),
-        int(window), int(keys_per_split), int(nsplit), _ptr(gate), gate_stride, int(gate_col),
-        float(out_scale), _stream())
+        int(window), int(chunk), int(keys_per_split), int(nsplit), _ptr(gate), gate_stride,
+        int(gate_col), 1 if gate_element else 0, float(out_scale), *extras, _stream())
     _check(rc, "paged_attention_gated")
     _note("attention", kernel="plain", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
 
 
-def head_gate_(out: torch.Tensor, gate: torch.Tensor, gate_col: int, out_scale: float = 1.0) -> torch.Tensor:
-    """``out [T, heads, width]`` times ``sigmoid(gate[t, gate_col + h]) * out_scale``, in place."""
+def head_gate_(out: torch.Tensor, gate: torch.Tensor, gate_col: int, out_scale: float = 1.0,
+               element: bool = False) -> torch.Tensor:
+    """``out [T, heads, width]`` times ``sigmoid(gate[t, gate_col + h]) * out_scale``, in place;
+    ``element``: times ``sigmoid(gate[t, gate_col + h * width + e]) * out_scale``."""
     T, nh, dv = out.shape
     _need(out, "out", (torch.float32, torch.bfloat16))
     _need(gate, "gate", out.dtype)
-    if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + nh > gate.shape[1]:
+    columns = nh * dv if element else nh
+    if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + columns > gate.shape[1]:
         raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
-                          f"{gate_col + nh} of {T} rows are needed")
-    rc = _fn("attention", "za_head_gate")(_ptr(out), _ptr(gate), _code(out.dtype), gate.shape[1],
-                                          int(gate_col), T, nh, dv, float(out_scale), _stream())
+                          f"{gate_col + columns} of {T} rows are needed")
+    rc = _fn("attention", "za_element_gate" if element else "za_head_gate")(
+        _ptr(out), _ptr(gate), _code(out.dtype), gate.shape[1], int(gate_col), T, nh, dv,
+        float(out_scale), _stream())
     _check(rc, "head_gate")
     return out
 
@@ -1773,13 +1815,15 @@ def _state_window(state: torch.Tensor, offset: int, count: int, name: str) -> Tu
     return state.data_ptr() + 4 * offset, state.stride(0)
 
 
-def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
-                     state: torch.Tensor, state_offset: int, token_seq: torch.Tensor,
-                     seq_start: torch.Tensor, slot_id: torch.Tensor) -> torch.Tensor:
-    """``silu(bias + depth-wise causal convolution)`` of columns ``col0 .. col0 + C`` of
+def causal_conv(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
+                state: torch.Tensor, state_offset: int, token_seq: torch.Tensor,
+                seq_start: torch.Tensor, slot_id: torch.Tensor, activation: Optional[str] = "silu",
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``act(bias + depth-wise causal convolution)`` of columns ``col0 .. col0 + C`` of
     ``x [T, columns]`` with ``taps [C, L]`` (the last tap meets the current token); the
     ``L - 1`` inputs before a portion come from ``state[slot, state_offset + c*(L-1) + j]``,
-    which then takes the portion's last inputs.  Returns 32-bit ``[T, C]``."""
+    which then takes the portion's last inputs.  ``activation``: ``"silu"`` or None.
+    Returns ``[T, C]`` of ``out_dtype`` (32-bit, or bfloat16 for bfloat16 inputs)."""
     T, stride = x.shape
     _need(x, "x", (torch.float32, torch.bfloat16))
     C, L = taps.shape
@@ -1788,6 +1832,10 @@ def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optio
         raise KernelError(f"{L} taps: the convolution kernel takes 1 to {CONV_MAX_TAPS}")
     if col0 < 0 or col0 + C > stride:
         raise KernelError(f"columns {col0}..{col0 + C} of {stride}")
+    if activation not in (None, "silu"):
+        raise KernelError(f"activation must be silu or None, got {activation!r}")
+    if out_dtype not in (torch.float32, x.dtype):
+        raise KernelError(f"a convolution of {x.dtype} inputs cannot store {out_dtype}")
     if bias is not None:
         _need(bias, "bias", torch.float32, (C,))
     S = slot_id.numel()
@@ -1795,12 +1843,20 @@ def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optio
     _need(seq_start, "seq_start", torch.int32, (S + 1,))
     _need(slot_id, "slot_id", torch.int32, (S,))
     base, slot_stride = _state_window(state, state_offset, C * (L - 1), "state")
-    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
-    rc = _fn("recurrent", "za_causal_conv_silu")(
+    out = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    rc = _fn("recurrent", "za_causal_conv")(
         _ptr(x), _code(x.dtype), stride, int(col0), _ptr(taps), _ptr(bias), base, slot_stride,
-        _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(out), T, S, C, L, _stream())
-    _check(rc, "causal_conv_silu")
+        _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(out), _code(out_dtype),
+        1 if activation == "silu" else 0, T, S, C, L, _stream())
+    _check(rc, "causal_conv")
     return out
+
+
+def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
+                     state: torch.Tensor, state_offset: int, token_seq: torch.Tensor,
+                     seq_start: torch.Tensor, slot_id: torch.Tensor) -> torch.Tensor:
+    """``causal_conv`` followed by silu, as 32-bit ``[T, C]``."""
+    return causal_conv(x, col0, taps, bias, state, state_offset, token_seq, seq_start, slot_id)
 
 
 RECURRENCE_ROWS_PER_LANE = 16
@@ -1955,13 +2011,17 @@ def fixed_decay_recurrence_chunked(vectors: torch.Tensor, q_col: int, k_col: int
 
 def retention_prepare(proj: torch.Tensor, q_col: int, k_col: int, v_col: int,
                       positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, dk: int,
-                      dv: int, rotary_dim: int, k_scale: float) -> torch.Tensor:
+                      dv: int, rotary_dim: int, k_scale: float,
+                      activation: Optional[str] = None) -> torch.Tensor:
     """From an opening projection's rows ``proj [T, columns]`` (queries, keys and values of
     ``heads`` heads at the three columns) the 32-bit vectors of the fixed-decay recurrence,
     ``[T, q: heads*dk | k: heads*dk | v: heads*dv]``: the first ``rotary_dim`` elements of
     every query and key rotated by the token's position (element ``i`` with ``i +
-    rotary_dim/2``, angle ``position * inv_freq[i]``), the keys times ``k_scale``."""
+    rotary_dim/2``, angle ``position * inv_freq[i]``), the keys times ``k_scale``.  With
+    ``activation="silu"`` queries, keys and values pass silu first."""
     _need(proj, "proj", (torch.float32, torch.bfloat16))
+    if activation not in (None, "silu"):
+        raise KernelError(f"activation must be silu or None, got {activation!r}")
     if proj.dim() != 2:
         raise KernelError(f"proj must be [T, columns], got {tuple(proj.shape)}")
     T, stride = proj.shape
@@ -1975,10 +2035,10 @@ def retention_prepare(proj: torch.Tensor, q_col: int, k_col: int, v_col: int,
         if col < 0 or col + n > stride:
             raise KernelError(f"{name}: columns {col}..{col + n} of {stride}")
     out = torch.empty((T, 2 * heads * dk + heads * dv), dtype=torch.float32, device=proj.device)
-    rc = _fn("recurrent", "za_retention_prepare")(
+    rc = _fn("recurrent", "za_retention_prepare_act")(
         _ptr(proj), _code(proj.dtype), stride, int(q_col), int(k_col), int(v_col), _ptr(positions),
         _ptr(inv_freq) if rotary_dim else None, _ptr(out), T, heads, dk, dv, int(rotary_dim),
-        float(k_scale), _stream())
+        float(k_scale), 1 if activation == "silu" else 0, _stream())
     _check(rc, "retention_prepare")
     return out
 

@@ -27,6 +27,17 @@ position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``).
 ``values="keys"``: there is no value projection, a token's value is its key as projected
 (the key rows of the opening projection are there a second time, so whatever stores
 q | k | v rows finds the same numbers in the value columns).
+
+Further: ``gate="element"`` (a sigmoid gate for every element of every head's output,
+``gate_proj`` of ``num_heads * value_dim`` rows), ``chunk`` (positions are counted in chunks of
+that many from the sequence's start and a query sees the earlier keys of its own chunk only;
+0: none), ``sink_value`` (a number: every head's softmax denominator also holds its
+exponential, a sink with a fixed score and no tensor) and ``conv`` (the number of taps of a
+depth-wise causal convolution over time that q, k and v pass right behind their
+projection, before norm and rotation; tensors ``q_conv.weight``, ``k_conv.weight``,
+``v_conv.weight`` of ``[channels, taps]``, no bias, no activation; the last ``taps - 1``
+projected rows of a request are kept in its state slot, so the mixer needs pages and a
+state).  These go through the general attention kernel.
 """
 
 from __future__ import annotations
@@ -37,7 +48,8 @@ from typing import Any, Dict, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import (Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer)
+from .base import (Mixer, PagedNeed, PagedStateNeed, Runtime, StateNeed, TensorRule, lookup,
+                   register_mixer)
 from .feed_forward import fuse_rows, pad_rows
 
 # Cutting long contexts pays only when the launch would otherwise leave most of the
@@ -96,6 +108,13 @@ class GroupedQueryAttention(Mixer):
             rules["sink"] = TensorRule(((nh,),), role="bias")
         if params.get("gate") == "head":
             rules["gate_proj.weight"] = TensorRule(((nh, H),))
+        elif params.get("gate") == "element":
+            rules["gate_proj.weight"] = TensorRule(((nh * dv, H),))
+        taps = int(params.get("conv") or 0)
+        if taps:
+            rules["q_conv.weight"] = TensorRule(((nh * d, taps),), role="filter")
+            rules["k_conv.weight"] = TensorRule(((nkv * d, taps),), role="filter")
+            rules["v_conv.weight"] = TensorRule(((nkv * dv, taps),), role="filter")
         if params.get("qk_norm"):
             rules["q_norm.weight"] = TensorRule(((d,),), role="norm")
             rules["k_norm.weight"] = TensorRule(((d,),), role="norm")
@@ -112,8 +131,15 @@ class GroupedQueryAttention(Mixer):
         nkv, d = int(params["num_kv_heads"]), int(params["head_dim"])
         dv = int(params.get("value_dim") or d)
         if dv == d:
-            return PagedNeed.kv(nkv, d, int(params.get("window") or 0))
-        return PagedNeed(((nkv, d), (nkv, dv)), int(params.get("window") or 0))
+            paged = PagedNeed.kv(nkv, d, int(params.get("window") or 0))
+        else:
+            paged = PagedNeed(((nkv, d), (nkv, dv)), int(params.get("window") or 0))
+        taps = int(params.get("conv") or 0)
+        if not taps:
+            return paged
+        # the convolution's last inputs, [channel][taps - 1] 32-bit floats a request
+        channels = (int(params["num_heads"]) + nkv) * d + nkv * dv
+        return PagedStateNeed(paged, StateNeed((max(1, channels * (taps - 1)),)))
 
     def __init__(self, params, tensors, runtime: Runtime):
         super().__init__(params, tensors, runtime)
@@ -124,11 +150,20 @@ class GroupedQueryAttention(Mixer):
             raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} groups")
         self.group = self.num_heads // self.num_kv_heads
         self.value_dim = int(params.get("value_dim") or self.head_dim)
-        if params.get("gate") not in (None, "head"):
-            raise ValueError(f"attention gate must be None or 'head', got {params.get('gate')!r}")
-        self.gated = params.get("gate") == "head"
-        # values of their own width, or a gate: the kernels that take the cache as two planes
-        self.wide = self.gated or self.value_dim != self.head_dim
+        if params.get("gate") not in (None, "head", "element"):
+            raise ValueError(f"attention gate must be None, 'head' or 'element', got "
+                             f"{params.get('gate')!r}")
+        self.gated = params.get("gate") in ("head", "element")
+        self.gate_element = params.get("gate") == "element"
+        self.chunk = int(params.get("chunk") or 0)
+        self.taps = int(params.get("conv") or 0)
+        if self.chunk < 0 or self.taps < 0 or self.taps > ops.CONV_MAX_TAPS:
+            raise ValueError(f"chunk {self.chunk} and conv {self.taps}: neither negative, at most "
+                             f"{ops.CONV_MAX_TAPS} taps")
+        # values of their own width, a gate, chunks or a convolution: the kernels that take
+        # the cache as two planes
+        self.wide = self.gated or self.value_dim != self.head_dim or bool(self.chunk) \
+            or bool(self.taps) or params.get("sink_value") is not None
         if self.value_dim % 8 or self.value_dim > 256:
             raise ValueError(f"value_dim {self.value_dim} must be a multiple of 8, at most 256")
         if self.group > ops.ATTENTION_MAX_ROWS:
@@ -158,8 +193,13 @@ class GroupedQueryAttention(Mixer):
         if self.shared_values and (self.value_dim != self.head_dim or params.get("bias")):
             raise ValueError("values that are the keys have the keys' width and no bias")
         temperature = params.get("query_temperature")
-        self.shape = ops.ScoreShape(params.get("softcap") or 0.0,
-                                    tensors["sink"] if params.get("sink") else None,
+        sink = tensors["sink"] if params.get("sink") else None
+        if params.get("sink_value") is not None:
+            if sink is not None:
+                raise ValueError("a sink is a tensor or a fixed number, not both")
+            sink = torch.full((self.num_heads,), float(params["sink_value"]), dtype=torch.float32,
+                              device=runtime.device)
+        self.shape = ops.ScoreShape(params.get("softcap") or 0.0, sink,
                                     tuple(temperature) if temperature else None)
         opening = [tensors["q_proj.weight"], tensors["k_proj.weight"],
                    tensors["k_proj.weight" if self.shared_values else "v_proj.weight"]]
@@ -180,6 +220,10 @@ class GroupedQueryAttention(Mixer):
             b = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]])
             self.b_qkv = torch.cat([b, b.new_zeros((self.w_qkv.shape[0] - b.numel(),))]).contiguous()
             self.b_out = tensors.get("out_proj.bias")
+        self.conv_w = None
+        if self.taps:
+            self.conv_w = torch.cat([tensors["q_conv.weight"], tensors["k_conv.weight"],
+                                     tensors["v_conv.weight"]], dim=0).contiguous()
         self.q_norm = tensors.get("q_norm.weight") if params.get("qk_norm") else None
         self.k_norm = tensors.get("k_norm.weight") if params.get("qk_norm") else None
         pos = params.get("position")
@@ -195,9 +239,10 @@ class GroupedQueryAttention(Mixer):
             raise ValueError("an attention with value_dim or gate takes a rotary position "
                              "encoding or none")
         self.mfma = self.mfma and self.value_dim == self.head_dim
-        if self.shape and self.wide:
-            raise ValueError("a cap, a sink or a query temperature go with values of the keys' "
-                             "width and no gate")
+        if self.wide and (self.shape or self.chunk):
+            # the two-plane path's matrix-core calls know neither; the general kernel does
+            self.mfma = False
+            self.item_granularities = [self.rows_per_item]
         self.rotation_in_attention = (
             not self.wide and self.fused_rotation and runtime.dtype == torch.bfloat16
             and self.position.rotary_dim == self.head_dim and self.position.pairing != "adjacent")
@@ -300,16 +345,24 @@ class GroupedQueryAttention(Mixer):
         qkv = ops.linear(x, self.w_qkv, self.b_qkv, tune=self.runtime.tune)
         key_plane, value_plane = cache.planes
         rot = self.position.rotary_dim if self.position is not None else 0
+        gate = qkv if self.gated else None
+        if self.taps:
+            # q | k | v through the convolution over time (the gate's columns stay as they
+            # are); the request's state slot carries the last inputs from step to step
+            qkv = ops.causal_conv(qkv, 0, self.conv_w, None, cache.state, 0, step.token_seq,
+                                  step.seq_start, step.slot_id, activation=None,
+                                  out_dtype=qkv.dtype)
         q = ops.qk_norm_rope_kv_write_wide(
             qkv, step.positions, step.slot_mapping[cache.group], self.q_norm, self.k_norm,
             self.position.inv_freq if rot else None, key_plane, value_plane, nh, nkv, d, dv, rot,
             bool(rot) and self.position.pairing == "adjacent", self.eps, write_kv=cache.writes)
         table = step.block_tables[cache.group]
-        gate = qkv if self.gated else None
         # (ranges are cut at absolute key positions: behind a window nearly all of them
         # would be empty, so a windowed layer's contexts are never cut)
         def split(n_items, **kw):
-            return (0, 1) if self.window else plan_split(n_items, nkv, step.max_keys, **kw)
+            # (nor are a chunked layer's, for the same reason)
+            return (0, 1) if self.window or self.chunk \
+                else plan_split(n_items, nkv, step.max_keys, **kw)
         if self.mfma and cache.kv is not None and cache.kv.shape[3] % 4 == 0:
             if step.n_tokens > step.n_seqs:
                 items = step.attention_items(self.mfma_rows_per_item)
@@ -323,13 +376,15 @@ class GroupedQueryAttention(Mixer):
                                                     None, None, step.n_seqs, self.scale,
                                                     self.window, keys, nsplit)
             if gate is not None:
-                ops.head_gate_(o, gate, self.gate_col)
+                ops.head_gate_(o, gate, self.gate_col, element=self.gate_element)
         else:
             item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
             keys, nsplit = split(n_items)
             o = ops.paged_attention_gated(q, key_plane, value_plane, table, step.positions,
                                           item_seq, item_row0, item_count, n_items, self.scale,
-                                          self.window, keys, nsplit, gate, self.gate_col)
+                                          self.window, keys, nsplit, gate, self.gate_col,
+                                          shape=self.shape, chunk=self.chunk,
+                                          gate_element=self.gate_element)
         if getattr(step, "taps", None) is not None:
             step.taps["q"] = q.clone()
             step.taps["o"] = o.clone()

@@ -95,6 +95,17 @@ class StateNeed:
     init: float = 0.0
 
 
+@dataclass(frozen=True)
+class PagedStateNeed:
+    """A mixer that keeps something per token in pages AND a fixed-size state per request
+    (an attention whose projections pass a short convolution over time keeps keys and
+    values, and the convolution's last inputs).  Its ``CacheView`` has the paged need's
+    fields and ``state``."""
+
+    paged: PagedNeed
+    state: StateNeed
+
+
 # ------------------------------------------------------------------- runtime
 @dataclass
 class Runtime:

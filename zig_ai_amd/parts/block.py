@@ -81,6 +81,46 @@ class PreNormMixerBlock:
 register_arrangement(PreNormMixerBlock.kind, PreNormMixerBlock)
 
 
+class ParallelResidualBlock:
+    """One norm, and mixer and feed-forward side by side on its output:
+
+        h = norm(x);   y = x + (mixer(h) + feed_forward(h))
+
+    The mixer's result enters the 32-bit stream at once, the feed-forward's is left pending
+    for the norm that follows (which adds it while it reads the stream)."""
+
+    kind = "parallel_residual"
+    slots = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+
+    def __init__(self, parts):
+        self.parts = dict(parts)
+        self.norm = parts["norm"]
+        self.mixer = parts["mixer"]
+        self.feed_forward = parts.get("feed_forward")
+
+    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
+                cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        from ..kernels import ops
+        h = self.norm.add_forward(residual, pending)
+        # (both parts have read ``h``, a tensor of its own, before anything is added)
+        m = self.mixer.forward(h, step, cache)
+        f = self.feed_forward.forward(h, step) if self.feed_forward is not None else None
+        if m is not None:
+            ops.stream_add_(residual, m)
+        return residual, f
+
+
+class ParallelMixerBlock(ParallelResidualBlock):
+    """The same for a layer that has no feed-forward: ``y = x + mixer(norm(x))``."""
+
+    kind = "parallel_residual_no_ff"
+    slots = {"norm": "norm", "mixer": "mixer"}
+
+
+register_arrangement(ParallelResidualBlock.kind, ParallelResidualBlock)
+register_arrangement(ParallelMixerBlock.kind, ParallelMixerBlock)
+
+
 class ScaledResidualBlock:
     """A pre-norm block whose parts enter the stream with weights, and which may run two
     mixers side by side on the same normed input and may lack the feed-forward:

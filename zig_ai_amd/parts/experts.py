@@ -85,7 +85,8 @@ register_feed_forward(TableExperts.kind, TableExperts)
 class RoutedExperts(FeedForward):
     """Small gated experts of which a router picks ``top`` for every token:
 
-        z = Wr x;  s = softmax(z) over all router outputs  (``scores="sigmoid"``: sigmoid(z))
+        z = Wr x (+ ``router.bias`` with ``router_bias``: part of the logits, unlike the
+        correction);  s = softmax(z) over all router outputs  (``scores="sigmoid"``: sigmoid(z))
         the choice goes by s + correction (``correction``: a tensor, used for the choice
         only), among the outputs of the ``groups_kept`` best of ``groups`` equal groups of
         neighbouring outputs (a group counts by its largest choice score; ``groups = 0``: no
@@ -117,6 +118,8 @@ class RoutedExperts(FeedForward):
         rules = {"router.weight": TensorRule(((E + ident, H),))}
         if params.get("correction"):
             rules["correction"] = TensorRule(((E + ident,),), role="bias")
+        if params.get("router_bias"):
+            rules["router.bias"] = TensorRule(((E + ident,),), role="bias")
         for e in range(E):
             rules[f"experts.{e}.gate.weight"] = TensorRule(((I, H),))
             rules[f"experts.{e}.up.weight"] = TensorRule(((I, H),))
@@ -157,6 +160,10 @@ class RoutedExperts(FeedForward):
         if self.shared_gated:
             rows.append(tensors["shared.token_gate.weight"])
         self.w_router = ops.projection_weight(torch.cat(rows, dim=0).contiguous())
+        self.b_router = None
+        if params.get("router_bias"):
+            b = tensors["router.bias"]
+            self.b_router = torch.cat([b, b.new_zeros((self.w_router.shape[0] - b.numel(),))]).contiguous()
         self.gate_up = self.down = None
         if E:
             self.gate_up = TableExperts._stack(
@@ -172,7 +179,7 @@ class RoutedExperts(FeedForward):
     def forward(self, x, step):
         T = x.shape[0]
         tune = self.runtime.tune
-        logits = ops.linear(x, self.w_router, out_dtype=torch.float32, tune=tune)
+        logits = ops.linear(x, self.w_router, self.b_router, out_dtype=torch.float32, tune=tune)
         chosen, weight = ops.route_topk(logits, self.outputs, self.top, self.correction,
                                         self.groups, self.keep, self.route_scale, self.scores,
                                         self.renormalize)

@@ -130,5 +130,35 @@ class ClampedGLU(FeedForward):
         return ops.linear(a, self.down, tune=self.runtime.tune)
 
 
+class ActivatedMLP(FeedForward):
+    """A feed-forward without a gate: ``Wd act(Wu x)``, no biases.  ``activation``: ``relu2``,
+    the square of relu, taken in 32-bit by a kernel of its own."""
+
+    kind = "activated_mlp"
+    graph_safe = True
+    kernel_sources = ("gemm", "gemm_rows64", "activation")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, I = int(params["hidden_size"]), int(params["intermediate_size"])
+        return {"up.weight": TensorRule(((I, H),)), "down.weight": TensorRule(((H, I),))}
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.activation = str(params.get("activation", "relu2"))
+        if self.activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"feed-forward activation must be one of "
+                             f"{sorted(ops.UNARY_ACTIVATIONS)}, got {self.activation!r}")
+        self.up = ops.projection_weight(pad_rows(tensors["up.weight"]))
+        self.down = ops.projection_weight(pad_columns(tensors["down.weight"]))
+        ops.check_projection_weight(self.up, "feed_forward up")
+        ops.check_projection_weight(self.down, "feed_forward down")
+
+    def forward(self, x, step=None):
+        a = ops.activate(ops.linear(x, self.up, tune=self.runtime.tune), self.activation)
+        return ops.linear(a, self.down, out_dtype=torch.float32, tune=self.runtime.tune)
+
+
 register_feed_forward(SwiGLU.kind, SwiGLU)
 register_feed_forward(ClampedGLU.kind, ClampedGLU)
+register_feed_forward(ActivatedMLP.kind, ActivatedMLP)

@@ -35,6 +35,14 @@ multiplied by ``head_dim^-1/2``; per head ``h``
 then each head's ``o`` over its root mean square (``norm_eps``, no weight), times
 ``silu(g)``, and the output projection.  ``decay`` is a tuple of constants, one a head.
 The state slot holds ``S`` in 32-bit; what enters the walk (rotated q and k, v) is 32-bit.
+Four parameters turn it into other linear attentions of the same walk: ``activation``
+(``"silu"``: q, k and v pass silu right behind their projection; None), ``key_scale`` (what the
+keys are multiplied by; ``head_dim^-1/2`` unless given), ``output_norm`` (``"head"``: every
+head's read-out over its own root mean square, no weight; ``"all"``: the heads' read-outs
+side by side are normed together, times a weight ``norm.weight`` of ``num_heads * value_dim``)
+and ``gate`` (``"silu"`` or ``"sigmoid"`` of the gate's projection, applied behind the norm).
+Lightning attention is ``activation="silu"``, ``key_scale=1``, ``output_norm="all"``,
+``gate="sigmoid"`` and no position encoding.
 A step in which some request brings more than ``ops.RETENTION_CHUNK`` tokens walks its
 portions as chunks side by side (``ops.fixed_decay_recurrence_chunked``): with a constant
 decay the state is linear in what the tokens bring.
@@ -219,11 +227,14 @@ class Retention(Mixer):
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
         W, H, d, dv = cls._sizes(params)
-        return {"q_proj.weight": TensorRule(((H * d, W),)),
-                "k_proj.weight": TensorRule(((H * d, W),)),
-                "v_proj.weight": TensorRule(((H * dv, W),)),
-                "gate_proj.weight": TensorRule(((H * dv, W),)),
-                "out_proj.weight": TensorRule(((W, H * dv),))}
+        rules = {"q_proj.weight": TensorRule(((H * d, W),)),
+                 "k_proj.weight": TensorRule(((H * d, W),)),
+                 "v_proj.weight": TensorRule(((H * dv, W),)),
+                 "gate_proj.weight": TensorRule(((H * dv, W),)),
+                 "out_proj.weight": TensorRule(((W, H * dv),))}
+        if params.get("output_norm", "head") == "all":
+            rules["norm.weight"] = TensorRule(((H * dv,),), role="norm")
+        return rules
 
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
@@ -240,7 +251,15 @@ class Retention(Mixer):
         self.heads, self.head_dim, self.value_dim = H, d, dv
         self.eps = float(params["norm_eps"])
         self.decay = torch.tensor(decay, dtype=torch.float32, device=runtime.device)
-        self.k_scale = float(d) ** -0.5
+        scale = params.get("key_scale")
+        self.k_scale = float(d) ** -0.5 if scale is None else float(scale)
+        self.activation = params.get("activation")
+        self.output_norm = str(params.get("output_norm", "head"))
+        self.gate = str(params.get("gate", "silu"))
+        if self.activation not in (None, "silu") or self.output_norm not in ("head", "all") \
+                or self.gate not in ("silu", "sigmoid"):
+            raise ValueError(f"retention: activation {self.activation!r}, output_norm "
+                             f"{self.output_norm!r}, gate {self.gate!r}")
         pos = params.get("position")
         self.position = lookup("position", pos.kind)(pos.params, {}, runtime) if pos is not None \
             else None
@@ -254,7 +273,11 @@ class Retention(Mixer):
             tensors["gate_proj.weight"])))
         self.w_out = ops.projection_weight(tensors["out_proj.weight"])
         self.gate_col = 2 * H * d + H * dv
-        self.ones = torch.ones((1,), dtype=torch.float32, device=runtime.device)
+        if self.output_norm == "all":
+            self.norm_w, self.norm_group = tensors["norm.weight"], H * dv
+        else:
+            self.norm_w = torch.ones((1,), dtype=torch.float32, device=runtime.device)
+            self.norm_group = dv
         # long portions are walked in chunks side by side (the step's work items of that size)
         self.chunked = d <= ops.RETENTION_CHUNK_MAX_DK
         self.item_granularities = [ops.RETENTION_CHUNK] if self.chunked else []
@@ -267,7 +290,7 @@ class Retention(Mixer):
         vectors = ops.retention_prepare(
             z, 0, H * d, 2 * H * d, step.positions,
             self.position.inv_freq if self.rotary_dim else None, H, d, dv, self.rotary_dim,
-            self.k_scale)
+            self.k_scale, self.activation)
         items = step.attention_items(ops.RETENTION_CHUNK) if self.chunked else None
         if items is not None and items[3] > step.n_seqs:
             # some request brings more than a chunk: chunks side by side (a function of the
@@ -281,8 +304,8 @@ class Retention(Mixer):
         if getattr(step, "taps", None) is not None:
             step.taps["vectors"] = vectors.clone()
             step.taps["o"] = o.clone()
-        h = ops.gated_group_norm(o, z, self.gate_col, self.ones, dv, self.eps, "silu",
-                                 gate_first=False)
+        h = ops.gated_group_norm(o, z, self.gate_col, self.norm_w, self.norm_group, self.eps,
+                                 self.gate, gate_first=False)
         return ops.linear(h, self.w_out, tune=self.runtime.tune)
 
 

@@ -7,9 +7,17 @@ kernel does, /root/reference/src/cuda/layer_kernels.cu:353-365) or ``(2i, 2i+1)`
 for ``pairing="adjacent"`` (rope.zig:46-53).  ``rotary_dim < head_dim`` rotates
 only the leading elements.  The attention mixer applies the rotation inside its
 fused query/key kernel; this part only owns the constants.
+
+``scaling`` (optional; ``{"factor", "low", "high", "original"}``) rescales the frequencies
+by wavelength ``l = 2 pi / f``, in three bands: ``l < original / high`` keeps ``f``;
+``l > original / low`` takes ``f / factor``; between the two, with ``s = (original / l - low)
+/ (high - low)``, ``(1 - s) f / factor + s f``.  The table is made once, in double
+precision.
 """
 
 from __future__ import annotations
+
+import math
 
 import torch
 
@@ -36,6 +44,18 @@ class RotaryEmbedding(PositionEncoding):
         i = torch.arange(0, self.rotary_dim // 2, dtype=torch.float64)
         inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64),
                               2.0 * i / self.rotary_dim)
+        scaling = params.get("scaling")
+        if scaling:
+            factor, low, high, original = (float(scaling[k]) for k in
+                                           ("factor", "low", "high", "original"))
+            if factor <= 0.0 or high <= low or original <= 0.0:
+                raise ValueError(f"rope scaling needs factor > 0, high > low and original > 0, "
+                                 f"got {dict(scaling)!r}")
+            wave = 2.0 * math.pi / inv
+            blend = (original / wave - low) / (high - low)
+            middle = (1.0 - blend) * inv / factor + blend * inv
+            inv = torch.where(wave < original / high, inv,
+                              torch.where(wave > original / low, inv / factor, middle))
         self.inv_freq = inv.to(torch.float32).to(runtime.device)
 
 

@@ -8,6 +8,11 @@ Before pass ``row`` of the span the stream takes the row ``row`` of a table ``[p
 width]`` and, with ``add_origin``, the embedding's output once more:
 
     x <- x (+ pending) (+ origin) + table[row]
+
+``pass_mix``: for the same kind of model, where each pass of the span starts from a
+projection of the stream and the embedding's output side by side:
+
+    x <- W [x (+ pending); origin]          W: [width, 2 width], the stream's half first
 """
 
 from __future__ import annotations
@@ -45,6 +50,39 @@ class PassOffset(Part):
 
 
 register_stream_step(PassOffset.kind, PassOffset)
+
+
+class PassMix(Part):
+    kind = "pass_mix"
+    graph_safe = True
+    kernel_sources = ("norm", "gemm", "gemm_rows64", "activation")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        width = int(params["width"])
+        return {"weight": TensorRule(((width, 2 * width),))}
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.width = int(params["width"])
+        self.weight = ops.projection_weight(tensors["weight"])
+        ops.check_projection_weight(self.weight, "pass_mix weight")
+
+    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor],
+                origin: Optional[torch.Tensor], step):
+        if origin is None:
+            raise ValueError("the embedding's output was not kept for this model")
+        if pending is not None:
+            ops.stream_add_(residual, pending)
+        T, W = residual.shape
+        both = torch.empty((T, 2 * W), dtype=self.runtime.dtype, device=residual.device)
+        ops.copy_columns(residual, 0, W, both, 0)
+        ops.copy_columns(origin, 0, W, both, W)
+        # (a new stream: the product's 32-bit sums)
+        return ops.linear(both, self.weight, out_dtype=torch.float32, tune=self.runtime.tune), None
+
+
+register_stream_step(PassMix.kind, PassMix)
 
 
 class TokenSide(Part):
