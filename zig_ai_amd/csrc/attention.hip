@@ -39,12 +39,21 @@
 //                 and no value, neither scaled nor capped, counted once however the
 //                 context is cut (the kernel that sees the whole context adds it at its end,
 //                 otherwise the merge of the ranges does)
+//   chunks        positions are counted in chunks of `chunk` from the sequence's start, and
+//                 a query sees the keys of its own chunk only (chunk > 0); in the
+//                 matrix-core kernels the `SHAPED` instantiations know it
 struct ScoreExtras {
   float softcap;
   const float* sink;
   float qt_coef;
   int qt_every;
+  int chunk;
 };
+
+// first key a query at `position` sees when positions are counted in chunks (0 without)
+__device__ __forceinline__ int chunk_start(const ScoreExtras& ex, int position) {
+  return ex.chunk > 0 && position > 0 ? (position / ex.chunk) * ex.chunk : 0;
+}
 
 __device__ __forceinline__ float query_temperature(const ScoreExtras& ex, int position) {
   if (ex.qt_every <= 0) return 1.0f;
@@ -96,14 +105,12 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
                        float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv,
                        int d, int page_size, float scale, int window, int keys_per_split,
                        int nsplit, int dv, const T* __restrict__ gate, int gate_stride,
-                       int gate_col, float out_scale, ScoreExtras ex, int chunk, int gate_elem) {
+                       int gate_col, float out_scale, ScoreExtras ex, int gate_elem) {
   // `dv`: width of a value (keys and queries have `d`); a page holds the keys of all
   // heads, [kv_head][offset][d], then the values turned round, [kv_head][dv][offset].
   // `gate`: when given, head h of token t is multiplied by
   // sigmoid(gate[t * gate_stride + gate_col + h]) * out_scale; with `gate_elem` every
   // element dd of it by its own sigmoid(gate[t * gate_stride + gate_col + h * dv + dd]).
-  // `chunk` > 0: positions are counted in chunks of that many from the sequence's start,
-  // and a query sees the keys of its own chunk only.
   extern __shared__ float smem[];
   const int ldk = d + 1, ldv = dv + 1;
   const size_t page_elems = (size_t)nkv * page_size * (d + dv);
@@ -126,7 +133,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
   int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
-  if (chunk > 0 && (pos_first / chunk) * chunk > lo) lo = (pos_first / chunk) * chunk;
+  if (chunk_start(ex, pos_first) > lo) lo = chunk_start(ex, pos_first);
   const int hi = pos_last;  // inclusive
   int range_lo = z * keys_per_split;
   int range_hi = range_lo + keys_per_split - 1;
@@ -197,7 +204,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
         const int kp = tile0 + lane;
         bool valid = lane < KT && kp <= pos && kp <= range_hi && kp >= lo;
         if (window > 0 && kp <= pos - window) valid = false;
-        if (chunk > 0 && kp < (pos / chunk) * chunk) valid = false;
+        if (kp < chunk_start(ex, pos)) valid = false;
         float s = -INFINITY;
         if (lane < KT) {
           const float* qr = Qs + r * d;
@@ -465,7 +472,12 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
-  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  if (SHAPED && chunk_start(ex, pos_first) > lo) lo = chunk_start(ex, pos_first);
+  // (the first key of its chunk, per row of this lane: 0 without chunks)
+  [[maybe_unused]] int chunk_lo[NS];
+#pragma unroll
+  for (int c = 0; c < NS; ++c) chunk_lo[c] = SHAPED ? chunk_start(ex, pos_row[c]) : 0;
   // with nsplit > 1 this workgroup serves the keys of one range only (ranges are
   // multiples of the tile, so a tile lies in one range); its partial result is
   // merged with the others' by attention_combine_kernel
@@ -578,6 +590,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 
     bool wave_sees = wave_active && tile0 <= wave_hi;
     if (window > 0 && tile0 + KT - 1 <= wave_lo - window) wave_sees = false;
+    // (the wave's first row has the earliest chunk of its rows)
+    if (SHAPED && tile0 + KT - 1 < chunk_start(ex, wave_lo)) wave_sees = false;
     if (wave_sees) {
       const bf16_t* ks = Ks + buf * KT * LDK;
       const bf16_t* vt = Vt + buf * D * LDV;
@@ -597,7 +611,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
       }
       // a tile every key of which counts for every row of the wave needs no mask
       const bool needs_mask = !wave_full || tile0 + KT - 1 > wave_lo || tile0 < lo ||
-                              tile0 + KT - 1 > hi || (window > 0 && tile0 <= wave_hi - window);
+                              tile0 + KT - 1 > hi || (window > 0 && tile0 <= wave_hi - window) ||
+                              (SHAPED && tile0 < chunk_start(ex, wave_hi));
       bf16x8_t pf[NS][KK];
 #pragma unroll
       for (int c = 0; c < NS; ++c) {
@@ -615,6 +630,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
           int last = pos_row[c] < hi ? pos_row[c] : hi;
           int first = lo;
           if (window > 0 && pos_row[c] - window + 1 > first) first = pos_row[c] - window + 1;
+          if (SHAPED && chunk_lo[c] > first) first = chunk_lo[c];
           last -= tile0 + grp * 4;
           first -= tile0 + grp * 4;
           const bool below = __any(first > 0);   // does any lane have keys before its first?
@@ -901,7 +917,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   // at once, so that the kernel's start is two trips to memory (entries and positions
   // side by side, then keys and values) and not three.  A wave whose tile turns out to
   // lie beyond the context has loaded in vain (from inside the pool, as every load here).
-  const bool early = window == 0;
+  const bool early = window == 0 && !(SHAPED && ex.chunk > 0);
   if (early) {
     const int first_tile0 = (nsplit == 1 ? 0 : z * keys_per_split) + wave * AM_KT;
     if (ps_shift >= 4) load_entries(first_tile0);
@@ -913,7 +929,9 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const int pos_row = row_valid ? positions[tok] : -1;
   [[maybe_unused]] const ShapedRow row_mul =
       shaped_row(ex, SHAPED ? scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row) : 0.f);
-  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  if (SHAPED && chunk_start(ex, pos_first) > lo) lo = chunk_start(ex, pos_first);
+  [[maybe_unused]] const int chunk_lo = SHAPED ? chunk_start(ex, pos_row) : 0;
   const int hi = pos_last;
   int range_lo = z * keys_per_split;
   int range_hi = range_lo + keys_per_split - 1;
@@ -1055,6 +1073,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         const int kp = tile0 + (jb >> 1) * 32 + grp * 8 + (jb & 1) * 4 + i;
         bool valid = kp <= pos_row && kp >= lo && kp <= range_hi;
         if (window > 0 && kp <= pos_row - window) valid = false;
+        if (SHAPED && kp < chunk_lo) valid = false;
         const float v = valid ? (SHAPED ? shaped_score_log2(ex, s[jb][i], row_mul)
                                         : s[jb][i] * scale_log2e)
                               : -INFINITY;
@@ -1157,7 +1176,7 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
                             float* part_ml, int nh, int nkv, int d, int page_size, float scale,
                             int window, int keys_per_split, int nsplit, int dv, const void* gate,
                             int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                            int chunk, int gate_elem, hipStream_t stream) {
+                            int gate_elem, hipStream_t stream) {
   const size_t shmem = ((size_t)KT * (d + 1) + (size_t)KT * (dv + 1) + (size_t)AT_MAX_ROWS * d +
                         AT_WAVES * 64) * sizeof(float);
   auto kernel = paged_attention_kernel<T, KT>;
@@ -1172,7 +1191,7 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)kv,
                      block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, part_acc,
                      part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv,
-                     (const T*)gate, gate_stride, gate_col, out_scale, ex, chunk, gate_elem);
+                     (const T*)gate, gate_stride, gate_col, out_scale, ex, gate_elem);
   return za_launch_status();
 }
 
@@ -1236,7 +1255,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
                                int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                               hipStream_t stream, int chunk = 0, int gate_elem = 0);
+                               hipStream_t stream, int gate_elem = 0);
 
 // dtype codes: 0 = float32, 1 = bfloat16
 extern "C" int za_paged_attention(const void* q, void* out, const void* kv, const int* block_table,
@@ -1248,7 +1267,7 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, d, nullptr, 0, 0,
-                             1.0f, ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
+                             1.0f, ScoreExtras{0.f, nullptr, 0.f, 0, 0}, stream);
 }
 
 // The same with values of width `dv` (a page: keys [kv_head][offset][d], then values
@@ -1267,7 +1286,7 @@ extern "C" int za_paged_attention_gated(const void* q, void* out, const void* kv
   return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, dv, gate,
-                             gate_stride, gate_col, out_scale, ScoreExtras{0.f, nullptr, 0.f, 0},
+                             gate_stride, gate_col, out_scale, ScoreExtras{0.f, nullptr, 0.f, 0, 0},
                              stream);
 }
 
@@ -1281,13 +1300,13 @@ extern "C" int za_paged_attention_shaped(const void* q, void* out, const void* k
                                          int nh, int nkv, int d, int dv, int page_size, float scale,
                                          int window, int keys_per_split, int nsplit,
                                          float softcap, const float* sink, float qt_coef,
-                                         int qt_every, hipStream_t stream) {
-  if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D || softcap < 0.f || qt_every < 0)
+                                         int qt_every, int chunk, hipStream_t stream) {
+  if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D || softcap < 0.f || qt_every < 0 || chunk < 0)
     return ZA_ERR_UNSUPPORTED;
   return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, dv, nullptr, 0, 0,
-                             1.0f, ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
+                             1.0f, ScoreExtras{softcap, sink, qt_coef, qt_every, chunk}, stream);
 }
 
 static int paged_attention_any(const void* q, void* out, const void* kv, const int* block_table,
@@ -1297,9 +1316,9 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
                                int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
-                               hipStream_t stream, int chunk, int gate_elem) {
+                               hipStream_t stream, int gate_elem) {
   if (n_items == 0 || n_tokens == 0) return 0;
-  if (chunk < 0) return ZA_ERR_ARG;
+  if (ex.chunk < 0) return ZA_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || d <= 0 || page_size <= 0 ||
       bt_stride <= 0 || nsplit < 1 || !q || !out || !kv || !block_table || !positions ||
       !wi_seq || !wi_row0 || !wi_count)
@@ -1312,7 +1331,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
 #define ZA_AT_ARGS                                                                            \
   q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, part_acc, \
       part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv, gate,         \
-      gate_stride, gate_col, out_scale, ex, chunk, gate_elem, stream
+      gate_stride, gate_col, out_scale, ex, gate_elem, stream
   const bool small = d <= 128 && dv <= 128;
   if (dtype == 0) {
     rc = small ? launch_attention<float, 64>(ZA_AT_ARGS) : launch_attention<float, 32>(ZA_AT_ARGS);
@@ -1343,9 +1362,9 @@ extern "C" int za_paged_attention_general(
     const void* q, void* out, const void* kv, const int* block_table, int bt_stride,
     const int* positions, const int* wi_seq, const int* wi_row0, const int* wi_count, int n_items,
     int n_tokens, float* part_acc, float* part_ml, int dtype, int nh, int nkv, int d, int dv,
-    int page_size, float scale, int window, int chunk, int keys_per_split, int nsplit,
-    const void* gate, int gate_stride, int gate_col, int gate_elem, float out_scale, float softcap,
-    const float* sink, float qt_coef, int qt_every, hipStream_t stream) {
+    int page_size, float scale, int window, int keys_per_split, int nsplit, const void* gate,
+    int gate_stride, int gate_col, int gate_elem, float out_scale, float softcap,
+    const float* sink, float qt_coef, int qt_every, int chunk, hipStream_t stream) {
   if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D || softcap < 0.f || qt_every < 0 || chunk < 0)
     return ZA_ERR_UNSUPPORTED;
   if (gate && (gate_col < 0 || gate_col + (gate_elem ? nh * dv : nh) > gate_stride))
@@ -1354,7 +1373,7 @@ extern "C" int za_paged_attention_general(
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, dv, gate,
                              gate_stride, gate_col, out_scale,
-                             ScoreExtras{softcap, sink, qt_coef, qt_every}, stream, chunk,
+                             ScoreExtras{softcap, sink, qt_coef, qt_every, chunk}, stream,
                              gate_elem);
 }
 
@@ -1420,7 +1439,7 @@ static int attention_mfma_any(const void* q, void* out, const void* kv, const in
       part_acc, part_ml, nh, nkv, page_size, scale, window, keys_per_split, nsplit, ex, stream
   // tiles of 128 keys spread a tile's fixed work (running maximum, addresses) over twice
   // the scores: for long contexts; head size 128 keeps tiles of 64 (LDS)
-  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0) {
+  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0 || ex.chunk > 0) {
     if (d == 64) return tile_keys == 128 ? launch_attention_mfma<64, 128, true>(ZA_AM_ARGS)
                                          : launch_attention_mfma<64, 64, true>(ZA_AM_ARGS);
     return launch_attention_mfma<128, 64, true>(ZA_AM_ARGS);
@@ -1442,7 +1461,7 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
   return attention_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                             wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size,
                             scale, window, keys_per_split, nsplit, tile_keys,
-                            ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
+                            ScoreExtras{0.f, nullptr, 0.f, 0, 0}, stream);
 }
 
 // The same with what `ScoreExtras` describes.
@@ -1455,12 +1474,12 @@ extern "C" int za_paged_attention_mfma_shaped(const void* q, void* out, const vo
                                               int page_size, float scale, int window,
                                               int keys_per_split, int nsplit, int tile_keys,
                                               float softcap, const float* sink, float qt_coef,
-                                              int qt_every, hipStream_t stream) {
-  if (softcap < 0.f || qt_every < 0) return ZA_ERR_ARG;
+                                              int qt_every, int chunk, hipStream_t stream) {
+  if (softcap < 0.f || qt_every < 0 || chunk < 0) return ZA_ERR_ARG;
   return attention_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                             wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size,
                             scale, window, keys_per_split, nsplit, tile_keys,
-                            ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
+                            ScoreExtras{softcap, sink, qt_coef, qt_every, chunk}, stream);
 }
 
 template <bool ROPE, bool SHAPED = false>
@@ -1470,7 +1489,7 @@ static int launch_decode_mfma(const void* q, void* out, const void* kv, const in
                               float* part_acc, float* part_ml, int nh, int nkv, int d,
                               int page_size, float scale, int window, int keys_per_split,
                               int nsplit, const DecodeRope& rope, bool combine,
-                              hipStream_t stream, ScoreExtras ex = ScoreExtras{0.f, nullptr, 0.f, 0}) {
+                              hipStream_t stream, ScoreExtras ex = ScoreExtras{0.f, nullptr, 0.f, 0, 0}) {
   dim3 grid(n_items, nkv, nsplit), block(256);
   // Few workgroups (a small batch): eight waves each, so that a compute unit that
   // gets one workgroup still has eight waves' loads in flight.
@@ -1536,7 +1555,7 @@ static int decode_mfma_any(const void* q, void* out, const void* kv, const int* 
   if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
     return ZA_ERR_ARG;
   const DecodeRope none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
-  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0)
+  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0 || ex.chunk > 0)
     return launch_decode_mfma<false, true>(q, out, kv, block_table, bt_stride, positions, wi_seq,
                                            wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml,
                                            nh, nkv, d, page_size, scale, window, keys_per_split,
@@ -1558,7 +1577,7 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
                                               hipStream_t stream) {
   return decode_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
                          n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size, scale,
-                         window, keys_per_split, nsplit, ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
+                         window, keys_per_split, nsplit, ScoreExtras{0.f, nullptr, 0.f, 0, 0}, stream);
 }
 
 // The same with what `ScoreExtras` describes.
@@ -1567,12 +1586,12 @@ extern "C" int za_paged_attention_decode_mfma_shaped(
     const int* positions, const int* wi_seq, const int* wi_row0, const int* wi_count, int n_items,
     int n_tokens, float* part_acc, float* part_ml, int nh, int nkv, int d, int page_size,
     float scale, int window, int keys_per_split, int nsplit, float softcap, const float* sink,
-    float qt_coef, int qt_every, hipStream_t stream) {
-  if (softcap < 0.f || qt_every < 0) return ZA_ERR_ARG;
+    float qt_coef, int qt_every, int chunk, hipStream_t stream) {
+  if (softcap < 0.f || qt_every < 0 || chunk < 0) return ZA_ERR_ARG;
   return decode_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
                          n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size, scale,
                          window, keys_per_split, nsplit,
-                         ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
+                         ScoreExtras{softcap, sink, qt_coef, qt_every, chunk}, stream);
 }
 
 // The same for a step in which every request brings one token, with the token's part of

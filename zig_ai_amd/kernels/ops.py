@@ -134,8 +134,8 @@ _SIGNATURES = {
     ("attention", "za_paged_attention_general"): [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-        c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p, c_float,
-        c_int, c_void_p],
+        c_int, c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p, c_float,
+        c_int, c_int, c_void_p],
     ("recurrent", "za_retention_prepare"): [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
                                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                             c_float, c_void_p],
@@ -143,15 +143,15 @@ _SIGNATURES = {
                                                  c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                  c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                                  c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-                                                 c_float, c_void_p, c_float, c_int, c_void_p],
+                                                 c_float, c_void_p, c_float, c_int, c_int, c_void_p],
     ("attention", "za_paged_attention_mfma_shaped"): [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-        c_int, c_float, c_void_p, c_float, c_int, c_void_p],
+        c_int, c_float, c_void_p, c_float, c_int, c_int, c_void_p],
     ("attention", "za_paged_attention_decode_mfma_shaped"): [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-        c_float, c_void_p, c_float, c_int, c_void_p],
+        c_float, c_void_p, c_float, c_int, c_int, c_void_p],
     ("recurrent", "za_retention_chunked"): [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                             c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -1064,10 +1064,10 @@ class ScoreShape:
     def args(self, num_heads: int):
         if self.sink is not None:
             _need(self.sink, "sink", torch.float32, (num_heads,))
-        return self.softcap, _ptr(self.sink), self.coef, self.every
+        return self.softcap, _ptr(self.sink), self.coef, self.every, self.chunk
 
     def __bool__(self) -> bool:
-        return bool(self.softcap or self.sink is not None or self.every)
+        return bool(self.softcap or self.sink is not None or self.every or self.chunk)
 
 
 def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
@@ -1726,14 +1726,13 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
                           n_items: int, scale: float, window: int = 0, keys_per_split: int = 0,
                           nsplit: int = 1, gate: Optional[torch.Tensor] = None, gate_col: int = 0,
                           out_scale: float = 1.0, shape: Optional[ScoreShape] = None,
-                          chunk: int = 0, gate_element: bool = False) -> torch.Tensor:
+                          gate_element: bool = False) -> torch.Tensor:
     """``paged_attention`` for values of their own width: ``q [T, heads, head_dim]``, the
     cache as a plane of keys and a plane of values (see ``qk_norm_rope_kv_write_wide``);
     returns ``[T, heads, value_dim]``.  With ``gate [T, columns]`` head ``h`` of token ``t``
     is multiplied by ``sigmoid(gate[t, gate_col + h]) * out_scale``, or with ``gate_element``
     its element ``e`` by ``sigmoid(gate[t, gate_col + h * value_dim + e]) * out_scale``.
-    ``shape``: see ``ScoreShape``.  ``chunk > 0``: a query sees the keys ``j`` with
-    ``j // chunk == position // chunk`` only (chunks counted from the sequence's start)."""
+    ``shape``: see ``ScoreShape``."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -1745,8 +1744,8 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
                           f"{ATTENTION_MAX_ROWS}")
     if d % 8 or dv % 8 or d > 256 or dv > 256:
         raise KernelError(f"head widths {d} and {dv} must be multiples of 8, at most 256")
-    if chunk < 0 or window < 0:
-        raise KernelError("window and chunk must not be negative")
+    if window < 0:
+        raise KernelError("a window must not be negative")
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [requests, max_pages]")
@@ -1770,12 +1769,12 @@ def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane:
             raise KernelError("keys_per_split must be a positive multiple of 64")
         part_acc = torch.empty((T, nh, nsplit, dv), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
-    extras = shape.args(nh) if shape else (0.0, None, 0.0, 0)
+    extras = shape.args(nh) if shape else (0.0, None, 0.0, 0, 0)
     rc = _fn("attention", "za_paged_attention_general")(
         _ptr(q), _ptr(out), _ptr(key_plane), _ptr(block_table), block_table.shape[1],
         _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
         _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, dv, page_size, float(scale),
-        int(window), int(chunk), int(keys_per_split), int(nsplit), _ptr(gate), gate_stride,
+        int(window), int(keys_per_split), int(nsplit), _ptr(gate), gate_stride,
         int(gate_col), 1 if gate_element else 0, float(out_scale), *extras, _stream())
     _check(rc, "paged_attention_gated")
     _note("attention", kernel="plain", rows=T, dtype=q.dtype, nsplit=int(nsplit))

@@ -200,7 +200,7 @@ class GroupedQueryAttention(Mixer):
             sink = torch.full((self.num_heads,), float(params["sink_value"]), dtype=torch.float32,
                               device=runtime.device)
         self.shape = ops.ScoreShape(params.get("softcap") or 0.0, sink,
-                                    tuple(temperature) if temperature else None)
+                                    tuple(temperature) if temperature else None, self.chunk)
         opening = [tensors["q_proj.weight"], tensors["k_proj.weight"],
                    tensors["k_proj.weight" if self.shared_values else "v_proj.weight"]]
         self.gate_col = (self.num_heads + self.num_kv_heads) * self.head_dim \
@@ -239,9 +239,7 @@ class GroupedQueryAttention(Mixer):
             raise ValueError("an attention with value_dim or gate takes a rotary position "
                              "encoding or none")
         self.mfma = self.mfma and self.value_dim == self.head_dim
-        if self.wide and (self.shape or self.chunk):
-            # the two-plane path's matrix-core calls know neither; the general kernel does
-            self.mfma = False
+        if not self.mfma:
             self.item_granularities = [self.rows_per_item]
         self.rotation_in_attention = (
             not self.wide and self.fused_rotation and runtime.dtype == torch.bfloat16
@@ -369,12 +367,12 @@ class GroupedQueryAttention(Mixer):
                 keys, nsplit = split(items[3], target=BUSY_WORKGROUPS)
                 o = ops.paged_attention_mfma(q, cache.kv, table, step.positions, *items,
                                              self.scale, self.window, keys, nsplit,
-                                             tile_keys=128 if d == 64 else 64)
+                                             tile_keys=128 if d == 64 else 64, shape=self.shape)
             else:
                 keys, nsplit = split(step.n_seqs)
                 o = ops.paged_attention_decode_mfma(q, cache.kv, table, step.positions, None,
                                                     None, None, step.n_seqs, self.scale,
-                                                    self.window, keys, nsplit)
+                                                    self.window, keys, nsplit, shape=self.shape)
             if gate is not None:
                 ops.head_gate_(o, gate, self.gate_col, element=self.gate_element)
         else:
@@ -383,8 +381,7 @@ class GroupedQueryAttention(Mixer):
             o = ops.paged_attention_gated(q, key_plane, value_plane, table, step.positions,
                                           item_seq, item_row0, item_count, n_items, self.scale,
                                           self.window, keys, nsplit, gate, self.gate_col,
-                                          shape=self.shape, chunk=self.chunk,
-                                          gate_element=self.gate_element)
+                                          shape=self.shape, gate_element=self.gate_element)
         if getattr(step, "taps", None) is not None:
             step.taps["q"] = q.clone()
             step.taps["o"] = o.clone()

@@ -86,8 +86,11 @@ class ParallelResidualBlock:
 
         h = norm(x);   y = x + (mixer(h) + feed_forward(h))
 
-    The mixer's result enters the 32-bit stream at once, the feed-forward's is left pending
-    for the norm that follows (which adds it while it reads the stream)."""
+    The norm runs as a kernel of its own, so both parts read a tensor that nothing adds to.
+    A part that sets ``takes_stream`` or ``accepts_stream`` is handed the stream as the keyword
+    ``stream`` and may add its result there itself (it then returns ``None``); what a part
+    returns instead is added here (the mixer's) or left pending for the norm that follows,
+    which adds it while it reads the stream (the feed-forward's)."""
 
     kind = "parallel_residual"
     slots = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
@@ -102,9 +105,18 @@ class ParallelResidualBlock:
                 cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         from ..kernels import ops
         h = self.norm.add_forward(residual, pending)
-        # (both parts have read ``h``, a tensor of its own, before anything is added)
-        m = self.mixer.forward(h, step, cache)
-        f = self.feed_forward.forward(h, step) if self.feed_forward is not None else None
+
+        def adds(part):
+            runtime = getattr(part, "runtime", None)
+            return (getattr(part, "takes_stream", False) or getattr(part, "accepts_stream", False)) \
+                and (runtime is None or getattr(runtime, "stream_additions", True))
+
+        m = self.mixer.forward(h, step, cache, stream=residual) if adds(self.mixer) \
+            else self.mixer.forward(h, step, cache)
+        f = None
+        if self.feed_forward is not None:
+            f = self.feed_forward.forward(h, step, stream=residual) if adds(self.feed_forward) \
+                else self.feed_forward.forward(h, step)
         if m is not None:
             ops.stream_add_(residual, m)
         return residual, f

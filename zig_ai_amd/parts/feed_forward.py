@@ -136,6 +136,7 @@ class ActivatedMLP(FeedForward):
 
     kind = "activated_mlp"
     graph_safe = True
+    accepts_stream = True     # ``forward`` takes ``stream`` and may add its result there
     kernel_sources = ("gemm", "gemm_rows64", "activation")
 
     @classmethod
@@ -154,9 +155,10 @@ class ActivatedMLP(FeedForward):
         ops.check_projection_weight(self.up, "feed_forward up")
         ops.check_projection_weight(self.down, "feed_forward down")
 
-    def forward(self, x, step=None):
+    def forward(self, x, step=None, stream: Optional[torch.Tensor] = None):
         a = ops.activate(ops.linear(x, self.up, tune=self.runtime.tune), self.activation)
-        return ops.linear(a, self.down, out_dtype=torch.float32, tune=self.runtime.tune)
+        return ops.linear(a, self.down, out_dtype=torch.float32, accumulate=stream,
+                          tune=self.runtime.tune)
 
 
 register_feed_forward(SwiGLU.kind, SwiGLU)

@@ -218,6 +218,7 @@ class Retention(Mixer):
     kind = "retention"
     graph_safe = True
     takes_normed_rows = True      # ``x`` is only ever handed to ``ops.linear``
+    accepts_stream = True         # ``forward`` takes ``stream`` and may add its result there
     kernel_sources = ("gemm", "recurrent")
 
     @staticmethod
@@ -284,7 +285,7 @@ class Retention(Mixer):
         ops.check_projection_weight(self.w_in, "retention opening projection")
         ops.check_projection_weight(self.w_out, "retention out_proj")
 
-    def forward(self, x, step, cache):
+    def forward(self, x, step, cache, stream=None):
         H, d, dv = self.heads, self.head_dim, self.value_dim
         z = ops.linear(x, self.w_in, tune=self.runtime.tune)
         vectors = ops.retention_prepare(
@@ -306,7 +307,7 @@ class Retention(Mixer):
             step.taps["o"] = o.clone()
         h = ops.gated_group_norm(o, z, self.gate_col, self.norm_w, self.norm_group, self.eps,
                                  self.gate, gate_first=False)
-        return ops.linear(h, self.w_out, tune=self.runtime.tune)
+        return ops.linear(h, self.w_out, accumulate=stream, tune=self.runtime.tune)
 
 
 register_mixer(StateSpaceDuality.kind, StateSpaceDuality)
