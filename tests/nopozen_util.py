@@ -107,8 +107,9 @@ def make_tensors(cfg, seed=0):
     out = {"embed": normal(V, W), "final.norm": normal(W, std=0.3, mean=1.0),
            "head": normal(V, W, std=W ** -0.5)}
     if cfg.get("loop"):
-        out["loop.in"] = normal(W, 2 * W, std=(2 * W) ** -0.5) \
+        mix = normal(W, 2 * W, std=(2 * W) ** -0.5) \
             + torch.cat([torch.eye(W), torch.zeros(W, W)], dim=1) * 0.5
+        out["loop.in"] = mix.to(torch.bfloat16).to(torch.float32)
     for i, lay in enumerate(cfg["layers"]):
         p, m = f"l{i}.", lay["mixer"]
         out[p + "norm1"] = normal(W, std=0.3, mean=1.0)

@@ -1050,12 +1050,17 @@ class ScoreShape:
     ``softcap`` (``s <- softcap * tanh(s / softcap)`` after the scale; 0: none), ``sink``
     (32-bit ``[heads]``: ``exp(sink[h])`` joins the softmax's denominator once, with no key
     and no value; None: none) and ``temperature`` (``(coef, every)``: the query at position
-    ``p`` counts ``1 + coef * ln(floor((p + 1) / every) + 1)`` times; None: none)."""
+    ``p`` counts ``1 + coef * ln(floor((p + 1) / every) + 1)`` times; None: none); and to the
+    mask, ``chunk``: positions are counted in chunks of that many from the sequence's start
+    and a query sees the earlier keys of its own chunk only (0: every earlier key)."""
 
     def __init__(self, softcap: float = 0.0, sink: Optional[torch.Tensor] = None,
-                 temperature: Optional[Tuple[float, int]] = None):
+                 temperature: Optional[Tuple[float, int]] = None, chunk: int = 0):
         self.softcap = float(softcap or 0.0)
         self.sink = sink
+        self.chunk = int(chunk or 0)
+        if self.chunk < 0:
+            raise KernelError("a chunk must not be negative")
         self.coef, self.every = (float(temperature[0]), int(temperature[1])) if temperature \
             else (0.0, 0)
         if self.softcap < 0.0 or self.every < 0:
