@@ -6,6 +6,7 @@
     python bench.py --workload compare                    # Rudilix beside LFM2 at equal sizes
     python bench.py --workload compare --compare-design ranesun   # Ranesun beside Rudilix
     python bench.py --workload compare --compare-design gemodra   # Gemodra beside Ranesun
+    python bench.py --workload compare --compare-design nopozen   # Nopozen beside Ranesun
 
 Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
@@ -41,6 +42,10 @@ depth and vocabulary, the closest design the engine has (recurrent and attention
 every fourth without positions; routed small experts with a shared one; a token input a
 layer) beside a Ranesun model of the same width, depth and vocabulary, the closest design
 the engine has (attention with sinks, experts of which a token uses a few).
+``--compare-design nopozen``: a Nopozen model (lightning, convolved and chunked attention layers
+in turn, parallel blocks, dense and routed feed-forwards, the first half of the layers a looped
+span) beside a Ranesun model of the same width, depth and vocabulary, the closest design the
+engine has (a fixed-decay linear attention, attention with sinks, small experts, a loop).
 """
 
 import argparse
@@ -213,10 +218,41 @@ def gemodra_shape(width, layers, vocab):
             "layers": out, "max_position_embeddings": 128000}
 
 
+def nopozen_shape(width, layers, vocab):
+    """Layer sizes in the manner of a real model of this design: lightning layers (heads of
+    128 x 128, decays spread from 1 - 2^-5 to 1 - 2^-12), attention_2 layers (heads of 64 in
+    groups of eight a key head, a filter of 4 taps, half of every head rotated) and attention
+    layers (heads of 128 in groups of four, chunks of 1,024 positions, frequencies rescaled)
+    in turn; feed-forwards in turn dense (four times the width) and eight experts of twice
+    the width of which a token uses two; the first half of the layers a looped span that
+    runs once."""
+    heads = width // 128
+    lightning = {"heads": heads, "dim": 128, "vdim": 128,
+                 "decay": [1.0 - 2.0 ** -(5 + 7 * h / max(1, heads - 1)) for h in range(heads)]}
+    q_heads = width // 64
+    attention_2 = {"heads": q_heads, "kv_heads": max(1, q_heads // 8), "dim": 64, "vdim": 64,
+                   "scale": 0.125, "conv": 4, "rot": {"dims": 32, "base": 1e6}}
+    attention = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
+                 "scale": 128 ** -0.5, "mask": {"size": 1024},
+                 "rot": {"dims": 128, "base": 5e5, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                                              "original": 8192}}}
+    dense = {"kind": "dense", "ff": 4 * width}
+    moe = {"kind": "moe", "expert": {"ff": 2 * width}, "router": {"experts": 8, "top": 2}}
+    kinds = [("lightning", lightning), ("attention_2", attention_2), ("lightning", lightning),
+             ("attention", attention)]
+    out = []
+    for i in range(layers):
+        kind, mixer = kinds[i % 4]
+        out.append({"type": kind, "mixer": mixer, "mlp": dense if (i // 2) % 2 == 0 else moe})
+    return {"architecture": "Nopozen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "loop": {"start": 0, "stop": max(1, layers // 2), "times": 1}, "layers": out,
+            "max_position_embeddings": 128000}
+
+
 def compare(widths, layers, batch, prompt_len, steps, warmup, design="rudilix", only=None) -> dict:
     """Prefill and decode throughput of Rudilix and of LFM2 at equal sizes, or
     (``design="ranesun"``) of Ranesun and of Rudilix, or (``design="gemodra"``) of Gemodra and
-    of Ranesun."""
+    of Ranesun, or (``design="nopozen"``) of Nopozen and of Ranesun."""
     import torch
     from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
     from zig_ai_amd.kernels import ops
@@ -305,10 +341,11 @@ def compare(widths, layers, batch, prompt_len, steps, warmup, design="rudilix", 
 
     result = {"workload": "compare", "dtype": "bf16", "data": "synthetic", "layers": layers,
               "batch": batch, "prompt_len": prompt_len, "steps": steps, "warmup": warmup, "widths": {}}
-    if design in ("ranesun", "gemodra"):
+    if design in ("ranesun", "gemodra", "nopozen"):
         for width in widths:
-            pair = {"ranesun": ranesun_shape, "rudilix": rudilix_shape} if design == "ranesun" \
-                else {"gemodra": gemodra_shape, "ranesun": ranesun_shape}
+            pair = {"ranesun": {"ranesun": ranesun_shape, "rudilix": rudilix_shape},
+                    "gemodra": {"gemodra": gemodra_shape, "ranesun": ranesun_shape},
+                    "nopozen": {"nopozen": nopozen_shape, "ranesun": ranesun_shape}}[design]
             result["widths"][str(width)] = {name: measure(shape(width, layers, vocab))
                                             for name, shape in pair.items()
                                             if only in (None, name)}
@@ -368,7 +405,8 @@ def main() -> int:
     ap.add_argument("--compare-widths", default="1024,2048",
                     help="--workload compare: the widths, with commas between them")
     ap.add_argument("--compare-layers", type=int, default=8, help="--workload compare: layers")
-    ap.add_argument("--compare-design", choices=["rudilix", "ranesun", "gemodra"], default="rudilix",
+    ap.add_argument("--compare-design", choices=["rudilix", "ranesun", "gemodra", "nopozen"],
+                    default="rudilix",
                     help="--workload compare: rudilix (beside LFM2), ranesun (beside Rudilix) or "
                          "gemodra (beside Ranesun)")
     ap.add_argument("--compare-only", default=None,
