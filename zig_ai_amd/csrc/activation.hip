@@ -287,6 +287,34 @@ extern "C" int za_activate(const void* in, void* out, int dtype, long long n, in
   return za_launch_status();
 }
 
+// out[r, c] = in[r, c] + bias[c]: the bias of a product whose 32-bit sums another kernel (or
+// a library) left, rounded once into the result's type.  `out` may be `in` for 32-bit results.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+bias_add_kernel(const float* __restrict__ in, const float* __restrict__ bias, TO* __restrict__ out,
+                size_t total, int N) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  out[idx] = from_f32<TO>(in[idx] + bias[idx % N]);
+}
+
+extern "C" int za_bias_add(const float* in, const float* bias, void* out, int out_dtype,
+                           long long rows, int N, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || N <= 0 || !in || !bias || !out) return ZA_ERR_ARG;
+  const size_t total = (size_t)rows * N;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (out_dtype == 0)
+    hipLaunchKernelGGL((bias_add_kernel<float>), grid, block, 0, stream, in, bias, (float*)out,
+                       total, N);
+  else if (out_dtype == 1)
+    hipLaunchKernelGGL((bias_add_kernel<bf16_t>), grid, block, 0, stream, in, bias, (bf16_t*)out,
+                       total, N);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}
+
 // x <- x * s, 32-bit, in place (an output head's constant factor on its logits).
 __global__ void __launch_bounds__(256) scale_kernel(float* __restrict__ x, float s, size_t n) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

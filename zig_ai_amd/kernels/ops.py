@@ -128,6 +128,7 @@ _SIGNATURES = {
     ("recurrent", "za_retention_prepare_act"): [c_void_p, c_int, c_int, c_int, c_int, c_int,
                                                 c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                                 c_int, c_int, c_float, c_int, c_void_p],
+    ("activation", "za_bias_add"): [c_void_p, c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
     ("activation", "za_activate"): [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
     ("attention", "za_element_gate"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                        c_int, c_float, c_void_p],
@@ -691,9 +692,9 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
-    ``LIBRARY_GEMM_ROWS`` rows (a decode batch), and always when a bias is asked
-    for; larger plain products go to the GEMM library, with bfloat16 or 32-bit
-    output.  32-bit weights use the all-32-bit kernel (``x`` may be either type and
+    ``LIBRARY_GEMM_ROWS`` rows (a decode batch); larger products go to the GEMM library,
+    with bfloat16 or 32-bit output (with a bias: the library's 32-bit sums, to which a small
+    kernel adds the bias before the one rounding).  32-bit weights use the all-32-bit kernel (``x`` may be either type and
     is widened): no library, no reduced-precision matrix mode.
 
     With ``partial_ok`` the result may come back as a stack ``[P, M, N]`` of 32-bit
@@ -815,8 +816,21 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
     # Many rows: the vendor's GEMM library, as the reference does for every
     # projection (/root/reference/src/matmul/root.zig:292-313 calls cuBLAS).
-    library = M > LIBRARY_GEMM_ROWS and bias is None and not force_tiled \
+    library = M > LIBRARY_GEMM_ROWS and not force_tiled \
         and out_dtype in (torch.bfloat16, torch.float32)
+    if library and bias is not None:
+        # the library's 32-bit sums, then the bias and one rounding by a small kernel
+        sums = _library_matmul(x, weight, torch.float32, 1, tune)
+        if sums is not None:
+            out = sums if out_dtype == torch.float32 else \
+                torch.empty((M, N), dtype=out_dtype, device=x.device)
+            rc = _fn("activation", "za_bias_add")(_ptr(sums), _ptr(bias), _ptr(out), _code(out_dtype),
+                                                  M, N, _stream())
+            _check(rc, "bias_add", f"M={M} N={N}")
+            _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False,
+                  partial_sums=1, out=out.dtype, kernel="library")
+            return out
+        library = False
     splits = 1
     if partial_ok and not force_tiled and K <= 8192 * 4 and (M <= 16 or library):
         splits = _k_splits(M, N, K)
