@@ -27,8 +27,9 @@ def rot(dims, base=300.0, scaling=None):
 
 def attention(heads=4, kv_heads=2, dim=16, vdim=None, scale=0.5, chunk=12, rot_dims=None,
               base=300.0, scaling=(4.0, 1.0, 3.0, 40)):
-    out = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim or dim, "scale": scale,
-           "rot": rot(rot_dims or dim, base, scaling)}
+    out = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim or dim, "scale": scale}
+    if rot_dims != 0:
+        out["rot"] = rot(rot_dims or dim, base, scaling)
     if chunk:
         out["mask"] = {"size": chunk}
     return out

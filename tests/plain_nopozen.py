@@ -114,12 +114,13 @@ def attention_mixer(h, p: str, W: Dict[str, torch.Tensor], m: dict, eps: float, 
     v = (h @ W[p + "v"].T + W[p + "v.b"]).view(T, G, dv)
     q = rms_norm(q, W[p + "q.norm"], eps)
     k = rms_norm(k, W[p + "k.norm"], eps)
-    q, k = rotate(q, positions, m["rot"]), rotate(k, positions, m["rot"])
+    if m.get("rot"):
+        q, k = rotate(q, positions, m["rot"]), rotate(k, positions, m["rot"])
     cache["k"] = k if "k" not in cache else torch.cat([cache["k"], k])
     cache["v"] = v if "v" not in cache else torch.cat([cache["v"], v])
     k_pos = torch.arange(cache["k"].shape[0])
     o = softmax_attention(q, cache["k"], cache["v"], positions, k_pos, float(m["scale"]),
-                          chunk=int(m["mask"]["size"]))
+                          chunk=int(m["mask"]["size"]) if m.get("mask") else 0)
     gate = torch.sigmoid(h @ W[p + "g"].T)                       # [T, H]
     o = o * gate[:, :, None]
     return o.reshape(T, H * dv) @ W[p + "o"].T + W[p + "o.b"]
@@ -212,8 +213,7 @@ class Walker:
         self.fed = 0
         self.dtype = dtype
 
-    def feed(self, tokens, without: str = ""):
-        """``without``: a mechanism to leave out (for tests that show it matters)."""
+    def feed(self, tokens):
         c, W = self.config, self.W
         eps = float(c["norm"]["eps"])
         ids = torch.as_tensor(tokens, dtype=torch.long)

@@ -70,6 +70,14 @@ ALONE = {
                                   rot_dims=16, scaling=(8.0, 1.0, 4.0, 64))),
     "attention, no frequency scaling, one chunk for all": nu.one_layer(
         "attention", nu.attention(heads=2, kv_heads=2, dim=24, chunk=4096, scaling=None)),
+    "attention, no rotation, no chunks": nu.one_layer(
+        "attention", nu.attention(heads=2, kv_heads=1, dim=16, chunk=0, rot_dims=0)),
+    "sizes that are multiples of nothing": nu.config([
+        nu.layer("attention", nu.attention(heads=3, kv_heads=1, dim=24, vdim=8, chunk=9, rot_dims=6),
+                 nu.dense(20)),
+        nu.layer("lightning", nu.lightning(heads=5, dim=12, vdim=20), nu.moe(ff=12, experts=7, top=3)),
+        nu.layer("attention_2", nu.attention_2(heads=3, kv_heads=3, dim=8, vdim=24, conv=2, rot_dims=6),
+                 nu.dense(44))], width=36, vocab=53, loop=(1, 3, 2)),
     "attention_2": nu.one_layer("attention_2", nu.attention_2()),
     "attention_2, one tap, whole rotation": nu.one_layer(
         "attention_2", nu.attention_2(heads=2, kv_heads=2, dim=16, vdim=16, conv=1, rot_dims=16)),
@@ -193,6 +201,21 @@ def test_schedules_bfloat16(which):
     for name, schedule in schedules(LENGTHS).items():
         peak = eu.peak_tokens(LENGTHS, schedule, round_to=16)
         got = eu.run_schedule(runner_for(model, page_size=16, tokens=peak), prompts, schedule)
+        assert_bfloat16_close(torch.cat(got), torch.cat(want), name)
+        base = base or got
+        assert_bfloat16_same(torch.cat(got), torch.cat(base), name)
+
+
+def test_sizes_that_are_multiples_of_nothing_in_bfloat16():
+    cfg = ALONE["sizes that are multiples of nothing"]
+    model, tensors = build(cfg, seed=13, dtype="bfloat16")
+    lengths = [60, 21, 2]
+    prompts = [nu.tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate(lengths)]
+    want = plain_logits(cfg, tensors, prompts)
+    base = None
+    for name, schedule in (("whole", eu.whole(lengths)), ("bulk + tail", eu.bulk_then_single(lengths, tail=20)),
+                           ("mixed", eu.mixed(lengths, seed=3, max_live=3, decode_tail=10))):
+        got = eu.run_schedule(runner_for(model, page_size=16, tokens=256), prompts, schedule)
         assert_bfloat16_close(torch.cat(got), torch.cat(want), name)
         base = base or got
         assert_bfloat16_same(torch.cat(got), torch.cat(base), name)

@@ -61,8 +61,12 @@ class RotarySizes:
 
     @classmethod
     def read(cls, m: Mapping[str, Any], dim: int, where: str) -> "RotarySizes":
+        if m.get("rot") is None:
+            return cls(0, 10000.0)                     # no rotation at all
         rot = _mapping(m, "rot", where)
-        dims = read_int(rot, ["dims"], minimum=2)
+        dims = read_int(rot, ["dims"], minimum=0)
+        if dims == 0:
+            return cls(0, read_float(rot, ["base"], default=10000.0, positive=True))
         if dims % 2 or dims > dim:
             raise ConfigError(f"{where}: rot.dims {dims} must be even and at most dim {dim}")
         scaling = None
@@ -82,7 +86,9 @@ class RotarySizes:
             out["scaling"] = dict(zip(("factor", "low", "high", "original"), self.scaling))
         return out
 
-    def spec(self, head_dim: int) -> PartSpec:
+    def spec(self, head_dim: int) -> Optional[PartSpec]:
+        if not self.dims:
+            return None
         params: Dict[str, Any] = {"head_dim": head_dim, "rotary_dim": self.dims,
                                   "theta": self.base, "pairing": "half"}
         if self.scaling:
@@ -145,7 +151,9 @@ class AttentionSizes:
 
     def to_dict(self) -> dict:
         out: Dict[str, Any] = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim,
-                               "vdim": self.vdim, "scale": self.scale, "rot": self.rot.to_dict()}
+                               "vdim": self.vdim, "scale": self.scale}
+        if self.rot.dims:
+            out["rot"] = self.rot.to_dict()
         if self.chunk:
             out["mask"] = {"size": self.chunk}
         if self.conv:
