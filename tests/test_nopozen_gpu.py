@@ -73,11 +73,13 @@ ALONE = {
     "attention, no rotation, no chunks": nu.one_layer(
         "attention", nu.attention(heads=2, kv_heads=1, dim=16, chunk=0, rot_dims=0)),
     "sizes that are multiples of nothing": nu.config([
-        nu.layer("attention", nu.attention(heads=3, kv_heads=1, dim=24, vdim=8, chunk=9, rot_dims=6),
+        nu.layer("attention", nu.attention(heads=3, kv_heads=1, dim=20, vdim=12, chunk=9, rot_dims=6),
                  nu.dense(20)),
         nu.layer("lightning", nu.lightning(heads=5, dim=12, vdim=20), nu.moe(ff=12, experts=7, top=3)),
-        nu.layer("attention_2", nu.attention_2(heads=3, kv_heads=3, dim=8, vdim=24, conv=2, rot_dims=6),
-                 nu.dense(44))], width=36, vocab=53, loop=(1, 3, 2)),
+        nu.layer("attention_2", nu.attention_2(heads=3, kv_heads=3, dim=10, vdim=28, conv=2, rot_dims=6),
+                 nu.dense(44)),
+        nu.layer("attention", nu.attention(heads=2, kv_heads=2, dim=6, vdim=6, chunk=4, rot_dims=6),
+                 None)], width=36, vocab=53, loop=(1, 3, 2)),
     "attention_2": nu.one_layer("attention_2", nu.attention_2()),
     "attention_2, one tap, whole rotation": nu.one_layer(
         "attention_2", nu.attention_2(heads=2, kv_heads=2, dim=16, vdim=16, conv=1, rot_dims=16)),

@@ -38,6 +38,13 @@ projection, before norm and rotation; tensors ``q_conv.weight``, ``k_conv.weight
 ``v_conv.weight`` of ``[channels, taps]``, no bias, no activation; the last ``taps - 1``
 projected rows of a request are kept in its state slot, so the mixer needs pages and a
 state).  These go through the general attention kernel.
+
+Head widths that are no multiple of 8 (what the kernels read at a time) are filled up with
+zeros when the part is built: zero rows of the q, k and v projections (and of their biases and
+filters), zero columns of the output projection; a score and a weighted sum do not change.
+The per-head norm then divides by the padded width: with ``eps * d / d_pad`` for eps and the
+norm's weight times ``sqrt(d / d_pad)`` the result is the same, ``x / sqrt(sum x^2 / d + eps) =
+sqrt(d / d_pad) x / sqrt(sum x^2 / d_pad + eps d / d_pad)``.
 """
 
 from __future__ import annotations
@@ -87,6 +94,20 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int, target: int = SPL
     return (keys, nsplit) if nsplit > 1 else (0, 1)
 
 
+def _round_up8(n: int) -> int:
+    return -(-int(n) // 8) * 8
+
+
+def _pad_heads(w: torch.Tensor, heads: int, width: int, padded: int) -> torch.Tensor:
+    """``w [heads * width, ...]`` -> ``[heads * padded, ...]``: zero rows behind every head's."""
+    if padded == width:
+        return w
+    rest = tuple(w.shape[1:])
+    w = w.reshape((heads, width) + rest)
+    return torch.cat([w, w.new_zeros((heads, padded - width) + rest)], dim=1) \
+        .reshape((heads * padded,) + rest).contiguous()
+
+
 class GroupedQueryAttention(Mixer):
     kind = "gqa_attention"
     graph_safe = True
@@ -129,7 +150,8 @@ class GroupedQueryAttention(Mixer):
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
         nkv, d = int(params["num_kv_heads"]), int(params["head_dim"])
-        dv = int(params.get("value_dim") or d)
+        dv = _round_up8(params.get("value_dim") or d)       # (as they lie in the cache: filled up)
+        d = _round_up8(d)
         if dv == d:
             paged = PagedNeed.kv(nkv, d, int(params.get("window") or 0))
         else:
@@ -145,11 +167,16 @@ class GroupedQueryAttention(Mixer):
         super().__init__(params, tensors, runtime)
         self.num_heads = int(params["num_heads"])
         self.num_kv_heads = int(params["num_kv_heads"])
-        self.head_dim = int(params["head_dim"])
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} groups")
         self.group = self.num_heads // self.num_kv_heads
-        self.value_dim = int(params.get("value_dim") or self.head_dim)
+        # the widths as the model has them, and as the kernels see them
+        self.model_head_dim = int(params["head_dim"])
+        self.model_value_dim = int(params.get("value_dim") or self.model_head_dim)
+        self.head_dim, self.value_dim = _round_up8(self.model_head_dim), _round_up8(self.model_value_dim)
+        norm_eps = float(params.get("norm_eps", 0.0))
+        if (self.head_dim, self.value_dim) != (self.model_head_dim, self.model_value_dim):
+            tensors, norm_eps = self._filled_up(params, tensors, norm_eps)
         if params.get("gate") not in (None, "head", "element"):
             raise ValueError(f"attention gate must be None, 'head' or 'element', got "
                              f"{params.get('gate')!r}")
@@ -179,14 +206,14 @@ class GroupedQueryAttention(Mixer):
         self.mfma_decode_rows_per_item = max(1, ops.ATTENTION_MFMA_DECODE_ROWS // self.group)
         self.window = int(params.get("window") or 0)
         scale = params.get("softmax_scale")
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.model_head_dim)
         # whether the matrix-core kernels take these sizes (the page size is checked per step)
         self.mfma = ops.attention_mfma_supported(runtime.dtype, self.num_heads,
                                                  self.num_kv_heads, self.head_dim,
                                                  scale=self.scale)
         self.item_granularities = [self.rows_per_item] + (
             [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
-        self.eps = float(params.get("norm_eps", 0.0))
+        self.eps = norm_eps
         if params.get("values") not in (None, "own", "keys"):
             raise ValueError(f"attention values must be 'own' or 'keys', got {params.get('values')!r}")
         self.shared_values = params.get("values") == "keys"
@@ -246,6 +273,27 @@ class GroupedQueryAttention(Mixer):
             and self.position.rotary_dim == self.head_dim and self.position.pairing != "adjacent")
         ops.check_projection_weight(self.w_qkv, "attention w_qkv")
         ops.check_projection_weight(self.w_out, "attention w_out")
+
+    def _filled_up(self, params, tensors, eps: float):
+        """The part's tensors with every head filled up with zeros to the kernels' widths, and
+        the eps that goes with the padded per-head norm."""
+        nh, nkv = self.num_heads, self.num_kv_heads
+        d0, dv0, d, dv = self.model_head_dim, self.model_value_dim, self.head_dim, self.value_dim
+        t = dict(tensors)
+        for name, heads, w0, w1 in (("q", nh, d0, d), ("k", nkv, d0, d), ("v", nkv, dv0, dv)):
+            for suffix in ("_proj.weight", "_proj.bias", "_conv.weight"):
+                if name + suffix in t:
+                    t[name + suffix] = _pad_heads(t[name + suffix], heads, w0, w1)
+        if params.get("gate") == "element":
+            t["gate_proj.weight"] = _pad_heads(t["gate_proj.weight"], nh, dv0, dv)
+        t["out_proj.weight"] = _pad_heads(t["out_proj.weight"].t().contiguous(), nh, dv0, dv) \
+            .t().contiguous()
+        if params.get("qk_norm"):
+            for name in ("q_norm.weight", "k_norm.weight"):
+                w = t[name].float() * math.sqrt(d0 / d)
+                t[name] = torch.cat([w, w.new_zeros((d - d0,))]).contiguous()
+            eps = eps * d0 / d
+        return t, eps
 
     def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
