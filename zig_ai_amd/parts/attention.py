@@ -37,7 +37,9 @@ depth-wise causal convolution over time that q, k and v pass right behind their
 projection, before norm and rotation; tensors ``q_conv.weight``, ``k_conv.weight``,
 ``v_conv.weight`` of ``[channels, taps]``, no bias, no activation; the last ``taps - 1``
 projected rows of a request are kept in its state slot, so the mixer needs pages and a
-state).  These go through the general attention kernel.
+state).  These go through the path that takes the cache as two planes: the matrix-core
+kernels where the sizes fit (the gate then is a small kernel behind them), the general
+attention kernel otherwise.
 
 Head widths that are no multiple of 8 (what the kernels read at a time) are filled up with
 zeros when the part is built: zero rows of the q, k and v projections (and of their biases and
