@@ -80,6 +80,10 @@ ALONE = {
                  nu.dense(44)),
         nu.layer("attention", nu.attention(heads=2, kv_heads=2, dim=6, vdim=6, chunk=4, rot_dims=6),
                  None)], width=36, vocab=53, loop=(1, 3, 2)),
+    "attention, forty heads on one key head": nu.one_layer(
+        "attention", nu.attention(heads=40, kv_heads=1, dim=8, vdim=8, chunk=30, rot_dims=4)),
+    "attention_2, sixty-six heads on two key heads": nu.one_layer(
+        "attention_2", nu.attention_2(heads=66, kv_heads=2, dim=8, vdim=8, conv=3, rot_dims=8)),
     "attention_2": nu.one_layer("attention_2", nu.attention_2()),
     "attention_2, one tap, whole rotation": nu.one_layer(
         "attention_2", nu.attention_2(heads=2, kv_heads=2, dim=16, vdim=16, conv=1, rot_dims=16)),

@@ -46,7 +46,9 @@ zeros when the part is built: zero rows of the q, k and v projections (and of th
 filters), zero columns of the output projection; a score and a weighted sum do not change.
 The per-head norm then divides by the padded width: with ``eps * d / d_pad`` for eps and the
 norm's weight times ``sqrt(d / d_pad)`` the result is the same, ``x / sqrt(sum x^2 / d + eps) =
-sqrt(d / d_pad) x / sqrt(sum x^2 / d_pad + eps d / d_pad)``.
+sqrt(d / d_pad) x / sqrt(sum x^2 / d_pad + eps d / d_pad)``.  More query heads a key head than a
+work item of the kernels holds (``ops.ATTENTION_MAX_ROWS``) are served by key heads that are
+there several times: the rows of the k and v projections are repeated until a group fits.
 """
 
 from __future__ import annotations
@@ -98,6 +100,25 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int, target: int = SPL
 
 def _round_up8(n: int) -> int:
     return -(-int(n) // 8) * 8
+
+
+def _kv_repeat(num_heads: int, num_kv_heads: int) -> int:
+    """How many times every key head is kept so that its group of query heads fits a work
+    item: the smallest divisor ``r`` of the group with ``group / r <= ATTENTION_MAX_ROWS``."""
+    group = num_heads // max(1, num_kv_heads)
+    for r in range(1, group + 1):
+        if group % r == 0 and group // r <= ops.ATTENTION_MAX_ROWS:
+            return r
+    return 1
+
+
+def _repeat_heads(w: torch.Tensor, heads: int, times: int) -> torch.Tensor:
+    """``w [heads * width, ...]`` with every head's rows ``times`` times in a row."""
+    if times == 1:
+        return w
+    rest = tuple(w.shape[1:])
+    return w.reshape((heads, -1) + rest).repeat_interleave(times, dim=0) \
+        .reshape((-1,) + rest).contiguous()
 
 
 def _pad_heads(w: torch.Tensor, heads: int, width: int, padded: int) -> torch.Tensor:
@@ -152,7 +173,8 @@ class GroupedQueryAttention(Mixer):
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
         nkv, d = int(params["num_kv_heads"]), int(params["head_dim"])
-        dv = _round_up8(params.get("value_dim") or d)       # (as they lie in the cache: filled up)
+        nkv *= _kv_repeat(int(params["num_heads"]), nkv)    # (as they lie in the cache)
+        dv = _round_up8(params.get("value_dim") or d)       # (filled up)
         d = _round_up8(d)
         if dv == d:
             paged = PagedNeed.kv(nkv, d, int(params.get("window") or 0))
@@ -179,6 +201,15 @@ class GroupedQueryAttention(Mixer):
         norm_eps = float(params.get("norm_eps", 0.0))
         if (self.head_dim, self.value_dim) != (self.model_head_dim, self.model_value_dim):
             tensors, norm_eps = self._filled_up(params, tensors, norm_eps)
+        repeat = _kv_repeat(self.num_heads, self.num_kv_heads)
+        if repeat > 1:
+            tensors = dict(tensors)
+            for name in ("k_proj.weight", "k_proj.bias", "k_conv.weight", "v_proj.weight",
+                         "v_proj.bias", "v_conv.weight"):
+                if name in tensors:
+                    tensors[name] = _repeat_heads(tensors[name], self.num_kv_heads, repeat)
+            self.num_kv_heads *= repeat
+            self.group //= repeat
         if params.get("gate") not in (None, "head", "element"):
             raise ValueError(f"attention gate must be None, 'head' or 'element', got "
                              f"{params.get('gate')!r}")
