@@ -207,3 +207,16 @@ def test_plain_walker_token_by_token():
     rows = [w.feed(prompt[:11])[0], w.feed(prompt[11:12])[0], w.feed(prompt[12:])[0]]
     assert torch.allclose(torch.cat(rows), whole, atol=1e-9)
     assert streams.shape == (11, 30, cfg["width"])
+
+
+def test_random_model_folder(tmp_path):
+    """The random model writer stores every tensor the design names, in the folder's format."""
+    from zig_ai_amd.weights import write_random_model
+    from zig_ai_amd.weights.safetensors_io import Checkpoint
+    cfg = config_from_dict(nu.TINY_ALL)
+    write_random_model(cfg, str(tmp_path), seed=3, dtype=torch.bfloat16)
+    ckpt = Checkpoint(str(tmp_path))
+    want = {k: tuple(v.shape) for k, v in nu.make_tensors(nu.TINY_ALL).items()}
+    assert {name: tuple(ckpt.shape(name)) for name in want} == want
+    from zig_ai_amd.config import load_config
+    assert load_config(str(tmp_path)) == cfg
